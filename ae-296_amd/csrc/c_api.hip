@@ -1,0 +1,322 @@
+// extern "C" surface of libmlora_hip.so (declared in include/mlora.h): argument
+// validation on the host, then one or two kernel launches on the caller's stream.
+// No allocation, no synchronisation, no state kept between calls.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/mlora.h"
+#include "mlora_args.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int log2_exact(int v)
+{
+    for (int s = 0; s < 31; s++)
+        if ((1 << s) == v) return s;
+    return -1;
+}
+
+int check_pool(mlora::PoolView &pv, const int32_t *a_tbl, const int32_t *b_tbl, const int32_t *rank,
+               const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages_a,
+               int64_t n_pages_b, int max_rank)
+{
+    if (!a_tbl || !b_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page tables, rank and scaling must not be NULL");
+    if (n_adapters <= 0) return fail(MLORA_EINVAL, "n_adapters must be positive (got %d)", n_adapters);
+    const int shift = log2_exact(page_rows);
+    if (shift < 0 || page_rows > 64) return fail(MLORA_EINVAL, "page_rows must be a power of two in 1..64 (got %d)", page_rows);
+    if (max_pages <= 0) return fail(MLORA_EINVAL, "max_pages must be positive (got %d)", max_pages);
+    if (max_rank < 1 || max_rank > MLORA_MAX_RANK) return fail(MLORA_ERANGE, "max_rank must be in 1..%d (got %d)", MLORA_MAX_RANK, max_rank);
+    if ((int64_t)max_pages * page_rows < max_rank)
+        return fail(MLORA_ERANGE, "max_pages * page_rows = %lld cannot hold max_rank %d", (long long)max_pages * page_rows, max_rank);
+    if (n_pages_a <= 0 || n_pages_b <= 0) return fail(MLORA_EINVAL, "n_pages_a / n_pages_b must be positive");
+    if (n_pages_a * page_rows > 0x7fffffffLL || n_pages_b * page_rows > 0x7fffffffLL)
+        return fail(MLORA_ERANGE, "a rows slab may hold at most 2^31-1 rows");
+    pv.a_tbl = a_tbl; pv.b_tbl = b_tbl; pv.rank = rank; pv.scaling = scaling;
+    pv.n_adapters = n_adapters; pv.max_pages = max_pages; pv.page_shift = shift;
+    pv.uniform_rank = 0; pv.uniform_scale = 0.f;
+    pv.n_rows_a = n_pages_a * page_rows; pv.n_rows_b = n_pages_b * page_rows;
+    pv.a_dense_stride = 0; pv.b_dense_stride = 0;
+    return MLORA_OK;
+}
+
+int check_dims(int hin, int hout)
+{
+    if (hin <= 0 || hout <= 0) return fail(MLORA_EINVAL, "hin and hout must be positive (got %d, %d)", hin, hout);
+    if ((hin & 7) || (hout & 7)) return fail(MLORA_EALIGN, "hin and hout must be multiples of 8 (got %d, %d)", hin, hout);
+    return MLORA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *mlora_last_error(void) { return g_err; }
+int mlora_version(void) { return 100; }
+
+int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
+                      const float *scaling, int n_adapters, int max_pages, int page_rows,
+                      int32_t *out_row_off, int32_t *out_rank, float *out_scale, int32_t *perm,
+                      int32_t *seg_start, int32_t *seg_len, int32_t *seg_adapter, int32_t *chunk_start,
+                      int32_t *chunk_len, int32_t *chunk_adapter, int group, int32_t *counters, void *stream)
+{
+    if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
+    if (T == 0) return MLORA_OK;
+    if (!tok_adapter) return fail(MLORA_EINVAL, "tok_adapter must not be NULL");
+    if (n_adapters <= 0 || n_adapters > (1 << 18)) return fail(MLORA_ERANGE, "n_adapters must be in 1..262144 (got %d)", n_adapters);
+    const bool per_tok = out_row_off || out_rank || out_scale;
+    if (per_tok) {
+        if (!page_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page_tbl, rank and scaling are needed for the per-token view");
+        if (max_pages <= 0 || page_rows <= 0) return fail(MLORA_EINVAL, "max_pages and page_rows must be positive");
+    }
+    const bool grouped = perm || seg_start || seg_len || seg_adapter || chunk_start || chunk_len || chunk_adapter || counters;
+    if (grouped) {
+        if (!(perm && seg_start && seg_len && seg_adapter && chunk_start && chunk_len && chunk_adapter && counters))
+            return fail(MLORA_EINVAL, "the grouped view needs all of perm, seg_*, chunk_* and counters");
+        if (T > MLORA_GATHER_MAX_T) return fail(MLORA_ERANGE, "T = %d exceeds MLORA_GATHER_MAX_T = %d", T, MLORA_GATHER_MAX_T);
+        if (group != 1 && group != 2 && group != 4 && group != 8) return fail(MLORA_EINVAL, "group must be 1, 2, 4 or 8 (got %d)", group);
+    }
+    if (!per_tok && !grouped) return MLORA_OK;
+    mlora::GatherArgs a;
+    a.tok_adapter = tok_adapter; a.page_tbl = page_tbl; a.rank = rank; a.scaling = scaling;
+    a.T = T; a.n_adapters = n_adapters; a.max_pages = max_pages > 0 ? max_pages : 1;
+    a.page_rows = page_rows > 0 ? page_rows : 1; a.group = grouped ? group : 1;
+    a.out_row_off = out_row_off; a.out_rank = out_rank; a.out_scale = out_scale;
+    a.perm = perm; a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter;
+    a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_adapter = chunk_adapter; a.counters = counters;
+    const int rc = mlora::launch_gather(a, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "gather launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+                     const void *const *b_rows, const int32_t *hin, const int32_t *hout,
+                     const int32_t *tok_adapter, int T, const int32_t *a_page_tbl, const int32_t *b_page_tbl,
+                     const int32_t *rank, const float *scaling, int n_adapters, int max_pages, int page_rows,
+                     int64_t n_pages_a, int64_t n_pages_b, int max_rank, const int32_t *perm,
+                     const int32_t *chunk_start, const int32_t *chunk_len, const int32_t *chunk_adapter,
+                     const int32_t *counters, int group, int dtype, int accumulate, void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
+    if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
+    if (T == 0) return MLORA_OK;
+    if (!y || !x || !a_rows || !b_rows || !hin || !hout) return fail(MLORA_EINVAL, "per-projection arrays must not be NULL");
+    if (!tok_adapter) return fail(MLORA_EINVAL, "tok_adapter must not be NULL");
+    mlora::BgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    int rc = check_pool(a.pool, a_page_tbl, b_page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank);
+    if (rc) return rc;
+    const bool grouped = perm != nullptr;
+    if (grouped) {
+        if (!(chunk_start && chunk_len && chunk_adapter && counters)) return fail(MLORA_EINVAL, "a grouped launch needs perm, chunk_* and counters");
+        if (group != 1 && group != 2 && group != 4 && group != 8) return fail(MLORA_EINVAL, "group must be 1, 2, 4 or 8 (got %d)", group);
+        if (group == 8 && max_rank > 32) return fail(MLORA_ERANGE, "group 8 supports max_rank <= 32 (got %d); use group 4", max_rank);
+    } else {
+        if (chunk_start || chunk_len || chunk_adapter) return fail(MLORA_EINVAL, "chunk arrays given without perm");
+        if (group != 1) return fail(MLORA_EINVAL, "group must be 1 when perm is NULL (got %d)", group);
+    }
+    for (int p = 0; p < n_proj; p++) {
+        if (!y[p] || !x[p] || !a_rows[p] || !b_rows[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
+        if (!aligned16(y[p]) || !aligned16(x[p]) || !aligned16(a_rows[p]) || !aligned16(b_rows[p]))
+            return fail(MLORA_EALIGN, "projection %d: device pointers must be 16-byte aligned", p);
+        rc = check_dims(hin[p], hout[p]);
+        if (rc) return rc;
+        a.y[p] = y[p]; a.x[p] = x[p]; a.a_rows[p] = a_rows[p]; a.b_rows[p] = b_rows[p];
+        a.hin[p] = hin[p]; a.hout[p] = hout[p];
+    }
+    a.tok_adapter = tok_adapter; a.tok_adapter64 = nullptr;
+    a.perm = perm; a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_adapter = chunk_adapter; a.counters = counters;
+    a.T = T; a.n_proj = n_proj; a.items_per_proj = T; a.accumulate = accumulate ? 1 : 0;
+    rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *tok_adapter,
+               const int32_t *a_page_tbl, const int32_t *b_page_tbl, const int32_t *rank, const float *scaling,
+               int T, int hin, int hout, int n_adapters, int max_pages, int page_rows, int64_t n_pages_a,
+               int64_t n_pages_b, int max_rank, int dtype, int accumulate, void *stream)
+{
+    void *ys[1] = {y};
+    const void *xs[1] = {x}, *as[1] = {a_rows}, *bs[1] = {b_rows};
+    const int32_t hi[1] = {hin}, ho[1] = {hout};
+    return mlora_bgmv_multi(1, ys, xs, as, bs, hi, ho, tok_adapter, T, a_page_tbl, b_page_tbl, rank, scaling,
+                            n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, 1, dtype, accumulate, stream);
+}
+
+int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const void *wb_T_all,
+                         const int64_t *indices, int T, int N, int L, int r, int hin, int hout, int layer_idx,
+                         float scale, int dtype, void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
+    if (T == 0) return MLORA_OK;
+    if (!y || !x || !wa_T_all || !wb_T_all || !indices) return fail(MLORA_EINVAL, "NULL device pointer");
+    if (N <= 0 || L <= 0) return fail(MLORA_EINVAL, "N and L must be positive (got %d, %d)", N, L);
+    if (layer_idx < 0 || layer_idx >= L) return fail(MLORA_ERANGE, "layer_idx %d outside [0, %d)", layer_idx, L);
+    if (r < 1 || r > MLORA_MAX_RANK) return fail(MLORA_ERANGE, "rank must be in 1..%d (got %d)", MLORA_MAX_RANK, r);
+    int rc = check_dims(hin, hout);
+    if (rc) return rc;
+    if (!aligned16(y) || !aligned16(x) || !aligned16(wa_T_all) || !aligned16(wb_T_all))
+        return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+    if ((int64_t)N * L * r > 0x7fffffffLL) return fail(MLORA_ERANGE, "pool has more than 2^31-1 rank rows");
+    mlora::BgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    mlora::PoolView &pv = a.pool;
+    pv.a_tbl = nullptr; pv.b_tbl = nullptr; pv.rank = nullptr; pv.scaling = nullptr;
+    pv.n_adapters = N; pv.max_pages = 1; pv.page_shift = 0;
+    pv.uniform_rank = r; pv.uniform_scale = scale;
+    // A: rank rows of adapter i, layer l start at row (i*L + l)*r; the layer offset goes into the base pointer.
+    pv.a_dense_stride = (long long)L * r;
+    pv.n_rows_a = (long long)(N - 1) * L * r + r;
+    // B^T: [hout, r] block of adapter i, layer l starts at element (i*L + l)*hout*r.
+    pv.b_dense_stride = (long long)L * hout * r;
+    pv.n_rows_b = 0;
+    a.y[0] = y; a.x[0] = x;
+    a.a_rows[0] = static_cast<const uint16_t *>(wa_T_all) + (size_t)layer_idx * r * hin;
+    a.b_rows[0] = static_cast<const uint16_t *>(wb_T_all) + (size_t)layer_idx * hout * r;
+    if (!aligned16(a.a_rows[0]) || !aligned16(a.b_rows[0]))
+        return fail(MLORA_EALIGN, "layer slab of the pool is not 16-byte aligned (r * hin and hout * r must be multiples of 8)");
+    a.hin[0] = hin; a.hout[0] = hout;
+    a.tok_adapter = nullptr; a.tok_adapter64 = indices;
+    a.T = T; a.n_proj = 1; a.items_per_proj = T; a.accumulate = 1;
+    rc = mlora::launch_bgmv(a, dtype, 1, r, true, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+}  // extern "C"
+
+namespace {
+
+constexpr int SG_TM = 64;   // tokens per tile, as in sgmv_prefill.hip
+
+struct SgmvWs { int max_tiles; int ksplit; size_t off_v, off_hi, off_lo, total; };
+
+SgmvWs sgmv_layout(int T, int n_seg)
+{
+    SgmvWs w;
+    w.max_tiles = T / SG_TM + n_seg + 1;
+    int ks = (1024 + w.max_tiles - 1) / w.max_tiles;
+    w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : ks);
+    size_t off = ((size_t)w.max_tiles * 3 + 4) * sizeof(int32_t);
+    off = (off + 255) & ~(size_t)255;
+    w.off_v = off;
+    off += (size_t)w.ksplit * T * MLORA_MAX_RANK * sizeof(float);
+    w.off_hi = off;
+    off += (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
+    w.off_lo = off;
+    off += (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
+    w.total = off;
+    return w;
+}
+
+void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
+{
+    char *base = static_cast<char *>(workspace);
+    int32_t *ip = reinterpret_cast<int32_t *>(base);
+    a.tile_seg = ip; a.tile_tok0 = ip + w.max_tiles; a.tile_ntok = ip + 2 * (size_t)w.max_tiles;
+    a.n_tiles = ip + 3 * (size_t)w.max_tiles;
+    a.v = reinterpret_cast<float *>(base + w.off_v);
+    a.vhi = reinterpret_cast<uint16_t *>(base + w.off_hi);
+    a.vlo = reinterpret_cast<uint16_t *>(base + w.off_lo);
+    a.max_tiles = w.max_tiles; a.ksplit = w.ksplit;
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t mlora_sgmv_workspace_bytes(int T, int n_seg)
+{
+    if (T <= 0 || n_seg <= 0) return 256;
+    return (int64_t)sgmv_layout(T, n_seg).total;
+}
+
+int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
+               const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *a_page_tbl,
+               const int32_t *b_page_tbl, const int32_t *rank, const float *scaling, int T, int hin, int hout,
+               int n_adapters, int max_pages, int page_rows, int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (T < 0 || n_seg < 0) return fail(MLORA_EINVAL, "T and n_seg must be >= 0 (got %d, %d)", T, n_seg);
+    if (T == 0 || n_seg == 0) return MLORA_OK;
+    if (!y || !x || !a_rows || !b_rows || !seg_start || !seg_len || !seg_adapter) return fail(MLORA_EINVAL, "NULL device pointer");
+    int rc = check_dims(hin, hout);
+    if (rc) return rc;
+    if (!aligned16(y) || !aligned16(x) || !aligned16(a_rows) || !aligned16(b_rows))
+        return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+    mlora::SgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = check_pool(a.pool, a_page_tbl, b_page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank);
+    if (rc) return rc;
+    const SgmvWs w = sgmv_layout(T, n_seg);
+    if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
+    if (workspace_bytes < (int64_t)w.total)
+        return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)w.total);
+    a.y = y; a.x = x; a.a_rows = a_rows; a.b_rows = b_rows;
+    a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter; a.n_seg = n_seg;
+    a.T = T; a.hin = hin; a.hout = hout; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0;
+    carve(a, workspace, w);
+    rc = mlora::launch_sgmv(a, dtype, max_rank, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "sgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void *B_T, int B, int Lpad, int L,
+                            int r, int hin, int hout, int layer_idx, int dtype, void *workspace,
+                            int64_t workspace_bytes, void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (B < 0 || Lpad < 0) return fail(MLORA_EINVAL, "B and Lpad must be >= 0 (got %d, %d)", B, Lpad);
+    if (B == 0 || Lpad == 0) return MLORA_OK;
+    if ((int64_t)B * Lpad > 0x7fffffffLL) return fail(MLORA_ERANGE, "B * Lpad exceeds 2^31-1 tokens");
+    if (!y || !x || !A_T || !B_T) return fail(MLORA_EINVAL, "NULL device pointer");
+    if (L <= 0 || layer_idx < 0 || layer_idx >= L) return fail(MLORA_ERANGE, "layer_idx %d outside [0, %d)", layer_idx, L);
+    if (r < 8 || r > MLORA_MAX_RANK || (r & 7)) return fail(MLORA_ERANGE, "prefill on the reference layout needs a rank that is a multiple of 8 in 8..%d (got %d)", MLORA_MAX_RANK, r);
+    int rc = check_dims(hin, hout);
+    if (rc) return rc;
+    if (!aligned16(y) || !aligned16(x) || !aligned16(A_T) || !aligned16(B_T))
+        return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+    if ((int64_t)B * L * r > 0x7fffffffLL) return fail(MLORA_ERANGE, "pool has more than 2^31-1 rank rows");
+    const int T = B * Lpad;
+    const SgmvWs w = sgmv_layout(T, B);
+    if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
+    if (workspace_bytes < (int64_t)w.total)
+        return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)w.total);
+    mlora::SgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    mlora::PoolView &pv = a.pool;
+    pv.n_adapters = B; pv.max_pages = 1; pv.page_shift = 0;
+    pv.uniform_rank = r; pv.uniform_scale = 1.0f;
+    pv.a_dense_stride = (long long)L * r;
+    pv.n_rows_a = (long long)(B - 1) * L * r + r;
+    pv.b_dense_stride = (long long)L * hout * r;
+    pv.n_rows_b = 0;
+    a.y = y; a.x = x;
+    a.a_rows = static_cast<const uint16_t *>(A_T) + (size_t)layer_idx * r * hin;
+    a.b_rows = static_cast<const uint16_t *>(B_T) + (size_t)layer_idx * hout * r;
+    a.n_seg = B; a.T = T; a.hin = hin; a.hout = hout; a.accumulate = 0; a.b_transposed = 1; a.seg_uniform_len = Lpad;
+    carve(a, workspace, w);
+    rc = mlora::launch_sgmv(a, dtype, r, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "prefill launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,95 @@
+// Kernel argument blocks and launcher prototypes shared between the kernels and
+// the C ABI layer.  Plain structs passed by value in the kernarg segment.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mlora {
+
+constexpr int MAX_PROJ = 8;
+constexpr int MAX_RANK = 64;
+
+// How the rank rows of an adapter are found inside a rows slab.
+struct PoolView {
+    const int32_t *a_tbl;      // [n_adapters, max_pages] or nullptr (dense)
+    const int32_t *b_tbl;
+    const int32_t *rank;       // [n_adapters] or nullptr (uniform_rank)
+    const float *scaling;      // [n_adapters] or nullptr (uniform_scale)
+    int n_adapters;
+    int max_pages;
+    int page_shift;            // log2(page_rows)
+    int uniform_rank;
+    float uniform_scale;
+    long long n_rows_a;        // slab extents in rows, for in-kernel bounds checks
+    long long n_rows_b;
+    long long a_dense_stride;  // rows between adapters when a_tbl == nullptr
+    long long b_dense_stride;  // rows (B as rank rows) or elements (B^T blocks) when b_tbl == nullptr
+};
+
+struct BgmvArgs {
+    void *y[MAX_PROJ];
+    const void *x[MAX_PROJ];
+    const void *a_rows[MAX_PROJ];
+    const void *b_rows[MAX_PROJ];
+    int hin[MAX_PROJ];
+    int hout[MAX_PROJ];
+    PoolView pool;
+    const int32_t *tok_adapter;    // [T] int32, or nullptr when tok_adapter64 is used
+    const int64_t *tok_adapter64;  // [T] int64 (reference layout call)
+    const int32_t *perm;           // grouped view (nullptr => one token per work item)
+    const int32_t *chunk_start;
+    const int32_t *chunk_len;
+    const int32_t *chunk_adapter;
+    const int32_t *counters;
+    int T;
+    int n_proj;
+    int items_per_proj;            // work-item bound per projection (T)
+    int accumulate;
+};
+
+struct GatherArgs {
+    const int32_t *tok_adapter;
+    const int32_t *page_tbl;
+    const int32_t *rank;
+    const float *scaling;
+    int T, n_adapters, max_pages, page_rows, group;
+    int32_t *out_row_off;
+    int32_t *out_rank;
+    float *out_scale;
+    int32_t *perm, *seg_start, *seg_len, *seg_adapter;
+    int32_t *chunk_start, *chunk_len, *chunk_adapter;
+    int32_t *counters;
+};
+
+struct SgmvArgs {
+    void *y;
+    const void *x;
+    const void *a_rows;
+    const void *b_rows;
+    PoolView pool;
+    const int32_t *seg_start;
+    const int32_t *seg_len;
+    const int32_t *seg_adapter;
+    int n_seg;
+    int T, hin, hout;
+    int accumulate;
+    int b_transposed;      // B given as [hout, r] blocks (reference layout)
+    int seg_uniform_len;   // > 0: segment s covers [s*len, (s+1)*len), adapter s (reference prefill)
+    // workspace carve-up
+    int32_t *tile_seg;     // [max_tiles]
+    int32_t *tile_tok0;
+    int32_t *tile_ntok;
+    int32_t *n_tiles;      // [1]
+    float *v;              // [ksplit, T, MAX_RANK] fp32 partial intermediates
+    uint16_t *vhi;         // [T, MAX_RANK] 16-bit hi part of the summed intermediate
+    uint16_t *vlo;         // [T, MAX_RANK] 16-bit lo part
+    int max_tiles;
+    int ksplit;
+};
+
+// launchers (defined next to their kernels); return hipError_t as int
+int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
+int launch_gather(const GatherArgs &a, hipStream_t s);
+int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, hipStream_t s);
+
+}  // namespace mlora

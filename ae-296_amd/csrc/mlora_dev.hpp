@@ -1,0 +1,113 @@
+// Device-side helpers shared by the gfx950 kernels: 16-byte vector access,
+// fp16/bf16 dot products with fp32 accumulation, and 16-lane DPP reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mlora {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf162_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf168_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+constexpr int DT_F16 = 0;
+constexpr int DT_BF16 = 1;
+
+__device__ __forceinline__ uint4 ldg16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+__device__ __forceinline__ void stg16(void *p, uint4 v) { *reinterpret_cast<uint4 *>(p) = v; }
+__device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
+
+// acc + sum_{e<2} a[e]*b[e], both 16-bit pairs packed in one dword, fp32 accumulate.
+template <int DT>
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc)
+{
+    if constexpr (DT == DT_F16) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, a), __builtin_bit_cast(half2_t, b), acc, false);
+    } else {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf162_t, a), __builtin_bit_cast(bf162_t, b), acc, false);
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ float dot8(const uint4 &a, const uint4 &b, float acc)
+{
+    acc = dot2<DT>(a.x, b.x, acc);
+    acc = dot2<DT>(a.y, b.y, acc);
+    acc = dot2<DT>(a.z, b.z, acc);
+    acc = dot2<DT>(a.w, b.w, acc);
+    return acc;
+}
+
+// low / high 16-bit lane of a dword as fp32
+template <int DT>
+__device__ __forceinline__ float lo_f32(uint32_t u)
+{
+    if constexpr (DT == DT_F16) return (float)__builtin_bit_cast(half2_t, u)[0];
+    else return __builtin_bit_cast(float, u << 16);
+}
+template <int DT>
+__device__ __forceinline__ float hi_f32(uint32_t u)
+{
+    if constexpr (DT == DT_F16) return (float)__builtin_bit_cast(half2_t, u)[1];
+    else return __builtin_bit_cast(float, u & 0xffff0000u);
+}
+
+template <int DT>
+__device__ __forceinline__ void unpack8(const uint4 &v, float (&f)[8])
+{
+    f[0] = lo_f32<DT>(v.x); f[1] = hi_f32<DT>(v.x);
+    f[2] = lo_f32<DT>(v.y); f[3] = hi_f32<DT>(v.y);
+    f[4] = lo_f32<DT>(v.z); f[5] = hi_f32<DT>(v.z);
+    f[6] = lo_f32<DT>(v.w); f[7] = hi_f32<DT>(v.w);
+}
+
+// fp32 -> 16-bit pattern, round to nearest even.
+template <int DT>
+__device__ __forceinline__ uint32_t cvt16(float f)
+{
+    if constexpr (DT == DT_F16) {
+        return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+    } else {
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x0040u;
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return u >> 16;
+    }
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi)
+{
+    return cvt16<DT>(lo) | (cvt16<DT>(hi) << 16);
+}
+
+template <int DT>
+__device__ __forceinline__ uint4 pack8(const float (&f)[8])
+{
+    return make_uint4(pack2<DT>(f[0], f[1]), pack2<DT>(f[2], f[3]), pack2<DT>(f[4], f[5]), pack2<DT>(f[6], f[7]));
+}
+
+// Sum over each aligned group of 16 lanes (a DPP "row"); every lane of the row gets the sum.
+__device__ __forceinline__ float row16_sum(float v)
+{
+    // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));
+    return v;
+}
+
+// Sum over the 64 lanes of a wavefront; every lane gets the sum.
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = row16_sum(v);
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+}  // namespace mlora

@@ -1,0 +1,218 @@
+// Adapter-pool index/offset gather for gfx950.
+//
+// Block 0 groups the tokens of a batch by adapter (stable: ordered by adapter id, then by
+// token id) with a bitonic sort of 32-bit keys in LDS, and derives segments and the decode
+// work list (chunks of at most `group` tokens of one adapter) with block-wide scans.
+// Blocks 1.. write the per-token view: page base rows, rank and scaling of each token's
+// adapter.  All outputs are integers or copied floats, so they are bit-exact by construction.
+//
+// Stands where the reference draws / selects its per-token index vector
+// (lightllm/models/lora_gpu.py:120,124,143,155) and drops the real per-request ids
+// (lightllm/server/router/model_infer/pre_process.py:50,100).
+#include "mlora_args.hpp"
+#include "mlora_dev.hpp"
+
+namespace mlora {
+
+constexpr int GATHER_NT = 1024;
+constexpr int GATHER_MAX_T = 8192;
+constexpr int TOK_BITS = 13;                 // token id field of the sort key
+constexpr int EPT = GATHER_MAX_T / GATHER_NT;  // sorted positions per thread in the scans
+
+// Inclusive scan over GATHER_NT per-thread values; op = 0 sum, 1 max, 2 min.
+template <int OP>
+__device__ __forceinline__ int scan_op(int a, int b)
+{
+    if constexpr (OP == 0) return a + b;
+    else if constexpr (OP == 1) return a > b ? a : b;
+    else return a < b ? a : b;
+}
+
+template <int OP>
+__device__ int block_scan_inclusive(int v, int identity, int *s_wave /* [16] */)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(v, d);
+        if (lane >= d) v = scan_op<OP>(v, o);
+    }
+    __syncthreads();                 // s_wave may still be read by a previous scan
+    if (lane == 63) s_wave[wave] = v;
+    __syncthreads();
+    int base = identity;
+    for (int w = 0; w < wave; w++) base = scan_op<OP>(base, s_wave[w]);
+    return scan_op<OP>(base, v);
+}
+
+__global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
+{
+    const int tid = threadIdx.x;
+    if (blockIdx.x > 0) {
+        // ---- per-token view
+        const long long idx = (long long)(blockIdx.x - 1) * GATHER_NT + tid;
+        const long long total = (long long)g.T * g.max_pages;
+        if (idx >= total) return;
+        const int t = (int)(idx / g.max_pages), pg = (int)(idx - (long long)t * g.max_pages);
+        int a = g.tok_adapter[t];
+        if (a >= g.n_adapters) a = -1;
+        int r = 0;
+        float s = 0.f;
+        int off = -1;
+        if (a >= 0) {
+            r = g.rank[a];
+            s = g.scaling[a];
+            const int np = (r + g.page_rows - 1) / g.page_rows;
+            if (pg < np) off = g.page_tbl[(long long)a * g.max_pages + pg] * g.page_rows;
+        }
+        if (g.out_row_off) g.out_row_off[idx] = off;
+        if (pg == 0) {
+            if (g.out_rank) g.out_rank[t] = r;
+            if (g.out_scale) g.out_scale[t] = s;
+        }
+        return;
+    }
+    if (!g.perm) return;
+
+    // ---- grouped view (one workgroup)
+    __shared__ uint32_t s_key[GATHER_MAX_T];
+    __shared__ int s_wave[16];
+    __shared__ int s_cnt[2];
+    const int T = g.T;
+    int n2 = 2;
+    while (n2 < T) n2 <<= 1;
+    if (tid < 2) s_cnt[tid] = 0;
+    __syncthreads();
+    const uint32_t sentinel = (uint32_t)g.n_adapters;   // "no adapter" sorts after every real adapter
+    for (int i = tid; i < n2; i += GATHER_NT) {
+        uint32_t key = 0xffffffffu;
+        bool valid = false, bad = false;
+        if (i < T) {
+            const int a = g.tok_adapter[i];
+            bad = a >= g.n_adapters;
+            valid = a >= 0 && !bad;
+            key = ((valid ? (uint32_t)a : sentinel) << TOK_BITS) | (uint32_t)i;
+        }
+        s_key[i] = key;
+        const unsigned long long mv = __ballot(valid), mb = __ballot(bad);
+        if ((tid & 63) == 0) {
+            if (mv) atomicAdd(&s_cnt[0], __popcll(mv));
+            if (mb) atomicAdd(&s_cnt[1], __popcll(mb));
+        }
+    }
+    __syncthreads();
+    for (int k = 2; k <= n2; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = tid; i < (n2 >> 1); i += GATHER_NT) {
+                const int lo = 2 * i - (i & (j - 1));
+                const int hi = lo + j;
+                const uint32_t a = s_key[lo], b = s_key[hi];
+                const bool up = (lo & k) == 0;
+                if ((a > b) == up) { s_key[lo] = b; s_key[hi] = a; }
+            }
+            __syncthreads();
+        }
+    }
+    const int n_valid = s_cnt[0];
+    const int gmask = g.group - 1;
+
+    // Each thread owns EPT consecutive sorted positions.
+    int ad[EPT], head[EPT];
+    const int base = tid * EPT;
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+        const int i = base + e;
+        ad[e] = -1; head[e] = 0;
+        if (i < T) {
+            const uint32_t key = s_key[i];
+            ad[e] = (int)(key >> TOK_BITS);
+            g.perm[i] = (int)(key & ((1u << TOK_BITS) - 1u));
+            head[e] = (i == 0) || ((int)(s_key[i - 1] >> TOK_BITS) != ad[e]);
+        }
+    }
+    // segment start of every position: running max of head positions
+    int run = 0, segstart[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; e++) { if (head[e]) run = base + e; segstart[e] = run; }
+    {
+        const int incl = block_scan_inclusive<1>(run, 0, s_wave);
+        const int prev = __shfl_up(incl, 1);          // exclusive value for this thread
+        __syncthreads();
+        if ((tid & 63) == 63) s_wave[tid >> 6] = incl;
+        __syncthreads();
+        int excl = (tid & 63) ? prev : ((tid >> 6) ? s_wave[(tid >> 6) - 1] : 0);
+        bool seen = false;
+#pragma unroll
+        for (int e = 0; e < EPT; e++) { seen = seen || head[e]; if (!seen) segstart[e] = excl; }
+    }
+    // segment end of every position: next head position after it (T if none): reverse running min
+    int segend[EPT];
+    {
+        int nxt = T;
+        int own_first = T;                       // first head position inside this thread's range
+#pragma unroll
+        for (int e = EPT - 1; e >= 0; e--) { segend[e] = nxt; if (head[e]) nxt = base + e; }
+        own_first = nxt;
+        // suffix min over threads = prefix min over reversed thread order
+        const int rt = GATHER_NT - 1 - tid;
+        __syncthreads();
+        __shared__ int s_first[GATHER_NT];
+        s_first[rt] = own_first;
+        __syncthreads();
+        const int mine = s_first[tid];            // value of thread (NT-1-tid)
+        const int incl = block_scan_inclusive<2>(mine, T, s_wave);
+        __syncthreads();
+        s_first[tid] = incl;                      // min over reversed index <= tid
+        __syncthreads();
+        const int after = rt > 0 ? s_first[rt - 1] : T;   // min over threads with larger tid
+#pragma unroll
+        for (int e = 0; e < EPT; e++) if (segend[e] == T) segend[e] = after < T ? after : T;
+    }
+    // running counts of real segment heads and of chunk heads
+    int nseg_local = 0, nch_local = 0, chead[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+        const int i = base + e;
+        chead[e] = (i < T) && (((i - segstart[e]) & gmask) == 0);
+        nseg_local += (head[e] && ad[e] < g.n_adapters) ? 1 : 0;
+        nch_local += chead[e];
+    }
+    const int seg_incl = block_scan_inclusive<0>(nseg_local, 0, s_wave);
+    const int ch_incl = block_scan_inclusive<0>(nch_local, 0, s_wave);
+    int seg_idx = seg_incl - nseg_local, ch_idx = ch_incl - nch_local;
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+        const int i = base + e;
+        const bool real = ad[e] >= 0 && ad[e] < g.n_adapters;
+        if (head[e] && real) {
+            g.seg_start[seg_idx] = i;
+            g.seg_len[seg_idx] = segend[e] - i;
+            g.seg_adapter[seg_idx] = ad[e];
+            seg_idx++;
+        }
+        if (chead[e]) {
+            const int left = segend[e] - i;
+            g.chunk_start[ch_idx] = i;
+            g.chunk_len[ch_idx] = left < g.group ? left : g.group;
+            g.chunk_adapter[ch_idx] = real ? ad[e] : -1;
+            ch_idx++;
+        }
+    }
+    if (tid == GATHER_NT - 1) {
+        g.counters[0] = seg_incl;
+        g.counters[1] = n_valid;
+        g.counters[2] = ch_incl;
+        g.counters[3] = s_cnt[1];
+        g.counters[4] = 0; g.counters[5] = 0; g.counters[6] = 0; g.counters[7] = 0;
+    }
+}
+
+int launch_gather(const GatherArgs &a, hipStream_t s)
+{
+    const long long per_tok = (a.out_row_off || a.out_rank || a.out_scale) ? (long long)a.T * a.max_pages : 0;
+    const unsigned grid = 1u + (unsigned)((per_tok + GATHER_NT - 1) / GATHER_NT);
+    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(GATHER_NT), 0, s, a);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mlora

@@ -1,0 +1,15 @@
+"""mlora: MI355X-native multi-LoRA batched apply (BGMV decode, SGMV prefill, adapter-pool gather).
+
+Host layer in Python over ``libmlora_hip.so`` (hand-written gfx950 kernels behind the C ABI of
+``include/mlora.h``).  Importing the package does not load the extension; the first call does,
+and raises if it has not been built.
+"""
+from . import _ext
+from ._ext import MloraError
+from .lora_gpu import Lora_GPU
+from .ops import (DecodePlan, add_lora_bgmv, bgmv, lora_apply, lora_prefill_ref, plan_decode, sgmv,
+                  sgmv_workspace)
+from .pool import AdapterPool
+
+__all__ = ["AdapterPool", "DecodePlan", "Lora_GPU", "MloraError", "add_lora_bgmv", "bgmv", "lora_apply",
+           "lora_prefill_ref", "plan_decode", "sgmv", "sgmv_workspace", "_ext"]

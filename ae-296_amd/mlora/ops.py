@@ -1,0 +1,234 @@
+"""Operator surface of the multi-LoRA apply path, on torch tensors in HBM.
+
+Three levels, all thin wrappers over the C ABI (``include/mlora.h``):
+
+* ``add_lora_bgmv`` -- signature-compatible stand-in for ``punica.ops.add_lora_bgmv`` as
+  the reference calls it (``lightllm/models/lora_gpu.py:138,150,162``), on the reference's
+  own pool layout; ``lora_prefill_ref`` likewise for the ``torch.bmm`` pair (``:127-128``).
+* ``plan_decode`` / ``bgmv`` / ``sgmv`` -- the paged-pool kernels.
+* ``lora_apply`` -- hidden states, per-token adapter index, pool, base projection output
+  to accumulate into.
+
+Every function launches on ``torch.cuda.current_stream()`` and returns without
+synchronising.  Nothing here computes on the CPU.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from . import _ext
+from .pool import AdapterPool
+
+_VoidArr = C.c_void_p * _ext.MAX_PROJ
+_IntArr = C.c_int32 * _ext.MAX_PROJ
+
+
+def _need_cuda(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("mlora kernels take device tensors; got a CPU tensor")
+
+
+def _need_contig(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_contiguous():
+            raise ValueError("mlora kernels take contiguous tensors")
+
+
+# ---------------------------------------------------------------------- gather / grouping
+@dataclass
+class DecodePlan:
+    """Device-side grouping of one decode batch by adapter (written by ``mlora_pool_gather``)."""
+    tok_adapter: torch.Tensor      # int32 [T]
+    group: int
+    perm: torch.Tensor             # int32 [T]
+    seg_start: torch.Tensor
+    seg_len: torch.Tensor
+    seg_adapter: torch.Tensor
+    chunk_start: torch.Tensor
+    chunk_len: torch.Tensor
+    chunk_adapter: torch.Tensor
+    counters: torch.Tensor         # int32 [8]: n_seg, n_valid, n_chunks, n_bad
+    row_off: Optional[torch.Tensor] = None   # int32 [T, max_pages]
+    tok_rank: Optional[torch.Tensor] = None
+    tok_scale: Optional[torch.Tensor] = None
+
+    @property
+    def T(self) -> int:
+        return self.tok_adapter.numel()
+
+
+def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: int = 4, per_token: bool = False,
+                out: Optional[DecodePlan] = None) -> DecodePlan:
+    """Index/offset gather for a decode batch: groups tokens by adapter (stable) and cuts the
+    groups into work items of at most `group` tokens.  Pass `out` to reuse a plan's buffers
+    (no allocation; safe under graph capture)."""
+    _need_cuda(tok_adapter)
+    if tok_adapter.dtype != torch.int32:
+        raise TypeError("tok_adapter must be int32")
+    _need_contig(tok_adapter)
+    T = tok_adapter.numel()
+    pool.sync()
+    dev = tok_adapter.device
+    if out is None:
+        i32 = dict(dtype=torch.int32, device=dev)
+        nseg = max(1, min(T, pool.n_slots))
+        out = DecodePlan(tok_adapter, group, torch.empty(max(T, 1), **i32), torch.empty(nseg, **i32),
+                         torch.empty(nseg, **i32), torch.empty(nseg, **i32), torch.empty(max(T, 1), **i32),
+                         torch.empty(max(T, 1), **i32), torch.empty(max(T, 1), **i32),
+                         torch.zeros(_ext.CNT_WORDS, **i32))
+        if per_token:
+            out.row_off = torch.empty((max(T, 1), pool.max_pages), **i32)
+            out.tok_rank = torch.empty(max(T, 1), **i32)
+            out.tok_scale = torch.empty(max(T, 1), dtype=torch.float32, device=dev)
+    else:
+        out.tok_adapter = tok_adapter
+        out.group = group
+    rc = _ext.lib().mlora_pool_gather(
+        _ext.ptr(tok_adapter), T, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
+        pool.n_slots, pool.max_pages, pool.page_rows,
+        _ext.ptr(out.row_off), _ext.ptr(out.tok_rank), _ext.ptr(out.tok_scale),
+        _ext.ptr(out.perm), _ext.ptr(out.seg_start), _ext.ptr(out.seg_len), _ext.ptr(out.seg_adapter),
+        _ext.ptr(out.chunk_start), _ext.ptr(out.chunk_len), _ext.ptr(out.chunk_adapter), group,
+        _ext.ptr(out.counters), _ext.current_stream_ptr())
+    _ext.check(rc)
+    return out
+
+
+# ---------------------------------------------------------------------- decode
+def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPool, layer: int,
+         projs: Sequence[str], tok_adapter: torch.Tensor, plan: Optional[DecodePlan] = None,
+         accumulate: bool = True) -> None:
+    """Decode LoRA apply for up to 8 projections of one layer in one launch:
+    ys[p][t] (+)= scaling[a] * (xs[p][t] . A_{p,a}) . B_{p,a},  a = tok_adapter[t]."""
+    n = len(projs)
+    if not (len(ys) == len(xs) == n) or not 1 <= n <= _ext.MAX_PROJ:
+        raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y and one x each")
+    _need_cuda(tok_adapter, *ys, *xs)
+    _need_contig(tok_adapter, *ys, *xs)
+    if tok_adapter.dtype != torch.int32:
+        raise TypeError("tok_adapter must be int32")
+    T = tok_adapter.numel()
+    yv, xv, av, bv, hi, ho = _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
+    for i, p in enumerate(projs):
+        hin, hout = pool.projections[p]
+        if xs[i].dtype != pool.dtype or ys[i].dtype != pool.dtype:
+            raise TypeError(f"x and y must have the pool dtype {pool.dtype}")
+        if tuple(xs[i].shape) != (T, hin) or tuple(ys[i].shape) != (T, hout):
+            raise ValueError(f"projection {p}: expected x [{T}, {hin}] and y [{T}, {hout}], "
+                             f"got {tuple(xs[i].shape)} and {tuple(ys[i].shape)}")
+        a_ptr, b_ptr = pool.slab_ptrs(layer, p)
+        yv[i], xv[i], av[i], bv[i], hi[i], ho[i] = ys[i].data_ptr(), xs[i].data_ptr(), a_ptr, b_ptr, hin, hout
+    pool.sync()
+    if plan is not None and plan.T != T:
+        raise ValueError("plan was built for a different batch size")
+    pp = plan
+    rc = _ext.lib().mlora_bgmv_multi(
+        n, yv, xv, av, bv, hi, ho, _ext.ptr(tok_adapter), T,
+        _ext.ptr(pool.page_tbl), _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
+        pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.n_pages, pool.max_rank,
+        _ext.ptr(pp.perm) if pp else None, _ext.ptr(pp.chunk_start) if pp else None,
+        _ext.ptr(pp.chunk_len) if pp else None, _ext.ptr(pp.chunk_adapter) if pp else None,
+        _ext.ptr(pp.counters) if pp else None, pp.group if pp else 1,
+        pool.dtype_code, int(accumulate), _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
+def add_lora_bgmv(y: torch.Tensor, x: torch.Tensor, wa_T_all: torch.Tensor, wb_T_all: torch.Tensor,
+                  indicies: torch.Tensor, layer_idx: int, scale: float) -> None:
+    """Same arguments and in-place semantics as ``punica.ops.add_lora_bgmv`` at the reference's
+    call sites (``lora_gpu.py:138,150,162``):
+        y[i] += x[i] @ wa_T_all[indicies[i], layer_idx].T @ wb_T_all[indicies[i], layer_idx].T * scale
+    with wa_T_all [N, L, r, Hin], wb_T_all [N, L, Hout, r], indicies int64 [B]."""
+    _need_cuda(y, x, wa_T_all, wb_T_all, indicies)
+    _need_contig(y, x, wa_T_all, wb_T_all, indicies)
+    if indicies.dtype != torch.int64:
+        raise TypeError("indicies must be int64 (as torch.randint produces at lora_gpu.py:120)")
+    if wa_T_all.dim() != 4 or wb_T_all.dim() != 4:
+        raise ValueError("wa_T_all must be [N, L, r, Hin] and wb_T_all [N, L, Hout, r]")
+    N, L, r, hin = wa_T_all.shape
+    N2, L2, hout, r2 = wb_T_all.shape
+    if (N2, L2, r2) != (N, L, r):
+        raise ValueError("wa_T_all and wb_T_all disagree on N, L or r")
+    T = x.shape[0]
+    if tuple(x.shape) != (T, hin) or tuple(y.shape) != (T, hout) or indicies.numel() != T:
+        raise ValueError("x must be [B, Hin], y [B, Hout], indicies [B]")
+    dt = _ext.dtype_code(x.dtype)
+    if not (y.dtype == x.dtype == wa_T_all.dtype == wb_T_all.dtype):
+        raise TypeError("y, x and the pool must share one 16-bit dtype")
+    rc = _ext.lib().mlora_bgmv_reflayout(y.data_ptr(), x.data_ptr(), wa_T_all.data_ptr(), wb_T_all.data_ptr(),
+                                         indicies.data_ptr(), T, N, L, r, hin, hout, layer_idx, float(scale), dt,
+                                         _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
+# ---------------------------------------------------------------------- prefill
+def sgmv_workspace(T: int, n_seg: int, device) -> torch.Tensor:
+    nbytes = _ext.lib().mlora_sgmv_workspace_bytes(T, n_seg)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: str,
+         seg_start: torch.Tensor, seg_len: torch.Tensor, seg_adapter: torch.Tensor,
+         accumulate: bool = True, workspace: Optional[torch.Tensor] = None) -> None:
+    """Prefill LoRA apply over packed segments (one adapter per segment) on MFMA tiles."""
+    _need_cuda(y, x, seg_start, seg_len, seg_adapter)
+    _need_contig(y, x, seg_start, seg_len, seg_adapter)
+    for s in (seg_start, seg_len, seg_adapter):
+        if s.dtype != torch.int32:
+            raise TypeError("segment arrays must be int32")
+    hin, hout = pool.projections[proj]
+    T = x.shape[0]
+    if tuple(x.shape) != (T, hin) or tuple(y.shape) != (T, hout):
+        raise ValueError(f"expected x [{T}, {hin}] and y [{T}, {hout}]")
+    if x.dtype != pool.dtype or y.dtype != pool.dtype:
+        raise TypeError(f"x and y must have the pool dtype {pool.dtype}")
+    n_seg = seg_start.numel()
+    if seg_len.numel() != n_seg or seg_adapter.numel() != n_seg:
+        raise ValueError("seg_start, seg_len and seg_adapter must have the same length")
+    if workspace is None:
+        workspace = sgmv_workspace(T, n_seg, x.device)
+    pool.sync()
+    a_ptr, b_ptr = pool.slab_ptrs(layer, proj)
+    rc = _ext.lib().mlora_sgmv(
+        y.data_ptr(), x.data_ptr(), a_ptr, b_ptr, seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(),
+        n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
+        T, hin, hout, pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.n_pages, pool.max_rank,
+        pool.dtype_code, int(accumulate), workspace.data_ptr(), workspace.numel(), _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
+def lora_prefill_ref(x: torch.Tensor, A_T: torch.Tensor, B_T: torch.Tensor, layer_idx: int,
+                     workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The reference's prefill expression on its own layout (``lora_gpu.py:125-128``):
+    ``torch.bmm(torch.bmm(x, A_T[:bsz, layer].transpose(-1,-2)), B_T[:bsz, layer].transpose(-1,-2))``
+    with x [bsz, Lpad, Hin], A_T [>=bsz, L, r, Hin], B_T [>=bsz, L, Hout, r]; request b uses slot b."""
+    _need_cuda(x, A_T, B_T)
+    _need_contig(x, A_T, B_T)
+    bsz, lpad, hin = x.shape
+    n, L, r, hin2 = A_T.shape
+    _, _, hout, _ = B_T.shape
+    if hin2 != hin or n < bsz or B_T.shape[0] < bsz or B_T.shape[1] != L or B_T.shape[3] != r:
+        raise ValueError("x, A_T and B_T shapes do not fit the reference prefill call")
+    if not (x.dtype == A_T.dtype == B_T.dtype):
+        raise TypeError("x and the pool must share one 16-bit dtype")
+    y = torch.empty((bsz, lpad, hout), dtype=x.dtype, device=x.device)
+    if workspace is None:
+        workspace = sgmv_workspace(bsz * lpad, bsz, x.device)
+    rc = _ext.lib().mlora_prefill_reflayout(y.data_ptr(), x.data_ptr(), A_T.data_ptr(), B_T.data_ptr(), bsz, lpad, L, r,
+                                            hin, hout, layer_idx, _ext.dtype_code(x.dtype), workspace.data_ptr(),
+                                            workspace.numel(), _ext.current_stream_ptr())
+    _ext.check(rc)
+    return y
+
+
+# ---------------------------------------------------------------------- one-call surface
+def lora_apply(y: torch.Tensor, x: torch.Tensor, tok_adapter: torch.Tensor, pool: AdapterPool, layer: int,
+               proj: str, plan: Optional[DecodePlan] = None) -> torch.Tensor:
+    """y (the base projection output, [T, Hout]) += LoRA delta of every token's adapter; returns y."""
+    bgmv([y], [x], pool, layer, [proj], tok_adapter, plan=plan, accumulate=True)
+    return y

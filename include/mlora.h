@@ -1,0 +1,178 @@
+/*
+ * mlora.h -- C ABI of libmlora_hip.so: multi-LoRA batched apply on MI355X (gfx950).
+ *
+ * The library replaces, for the LoRA-apply path only, what the reference reaches
+ * through two foreign interfaces:
+ *   - the third-party `punica.ops.add_lora_bgmv(y, x, wa_T_all, wb_T_all, indicies,
+ *     layer_idx, scale)` CUDA op called from lightllm/models/lora_gpu.py:138,150,162
+ *     (decode), and the `torch.bmm(torch.bmm(x, A), B)` pair at lora_gpu.py:127-128,
+ *     145-146,157-158 (prefill);
+ *   - nothing else: the copy helpers of the reference's own native module
+ *     (csrc/interface.cpp:18-79) belong to the CPU-assisted transport, not to this path.
+ *
+ * Conventions
+ *   - Every pointer named "device" is HIP device memory owned by the caller; the
+ *     library keeps no pointer between calls and allocates nothing.
+ *   - Calls are asynchronous on `stream` (a hipStream_t passed as void*, 0 = the
+ *     null stream) and may be captured into a HIP graph.
+ *   - 16-bit floats: dtype MLORA_F16 (IEEE binary16) or MLORA_BF16 (bfloat16);
+ *     all products are accumulated in fp32 and rounded once (nearest even) on store.
+ *   - Return value: MLORA_OK or a negative MLORA_E* code; mlora_last_error() then
+ *     returns a thread-local message.  Nothing throws or exits.
+ *   - Index validation that needs device data (adapter ids, page ids, ranks) is done
+ *     inside the kernels: an out-of-range adapter id is treated as "no adapter" and
+ *     counted in counters[MLORA_CNT_BAD]; an out-of-range page id contributes zero.
+ *     No kernel reads or writes outside the extents given here.
+ *
+ * Paged adapter pool (one slab per layer, projection and side)
+ *   rows      : [n_pages * page_rows, H] 16-bit floats, row-major, H % 8 == 0,
+ *               base 16-byte aligned.  An A slab holds rank rows of A^T (length Hin),
+ *               a B slab holds rank rows of B (length Hout).
+ *   page_tbl  : int32 [n_adapters, max_pages]; rank row j of adapter i is row
+ *               page_tbl[i][j / page_rows] * page_rows + j % page_rows.
+ *               page_rows is a power of two (1..64).  A NULL page table means the
+ *               dense layout: rank row j of adapter i is row i * dense_stride_rows + j.
+ *   rank      : int32 [n_adapters], 1..max_rank (max_rank <= 64).
+ *   scaling   : float [n_adapters]  (alpha / r).
+ *   tok_adapter : int32 [T]; a negative value means the token has no adapter.
+ */
+#ifndef MLORA_H
+#define MLORA_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLORA_OK 0
+#define MLORA_EINVAL (-1)   /* bad size / null pointer / unsupported combination */
+#define MLORA_ERANGE (-2)   /* value outside the supported range (rank, T, n_proj ...) */
+#define MLORA_EALIGN (-3)   /* pointer or row width not 16-byte aligned */
+#define MLORA_EDTYPE (-4)   /* dtype is neither MLORA_F16 nor MLORA_BF16 */
+#define MLORA_ELAUNCH (-5)  /* the HIP runtime refused the launch */
+#define MLORA_ENOSPACE (-6) /* caller-provided workspace too small */
+
+#define MLORA_F16 0
+#define MLORA_BF16 1
+
+#define MLORA_MAX_PROJ 8      /* projections batched in one decode launch */
+#define MLORA_MAX_RANK 64
+#define MLORA_GATHER_MAX_T 8192   /* tokens one mlora_pool_gather call can group */
+
+/* counters[] written by mlora_pool_gather (device int32[8]) */
+#define MLORA_CNT_NSEG 0     /* number of segments (distinct adapters present) */
+#define MLORA_CNT_NVALID 1   /* tokens that have an adapter */
+#define MLORA_CNT_NCHUNK 2   /* decode work items (chunks of <= group tokens of one adapter) */
+#define MLORA_CNT_BAD 3      /* tokens whose adapter id was >= n_adapters (treated as none) */
+#define MLORA_CNT_WORDS 8
+
+const char *mlora_last_error(void);
+int mlora_version(void);
+
+/*
+ * Adapter-pool index/offset gather + grouping of tokens by adapter.
+ * Replaces the per-token index vector the reference draws at lora_gpu.py:120 and
+ * selects at :124,143,155 (and the unused real ids of pre_process.py:50,100).
+ *
+ * Per-token view (each output may be NULL to skip it):
+ *   out_row_off [T, max_pages] = page_tbl[a][p] * page_rows for p < ceil(rank[a]/page_rows), else -1
+ *   out_rank [T], out_scale [T]                      (0 / 0.0f for tokens without adapter)
+ * Grouped view (all of perm..counters NULL to skip):
+ *   perm [T]            token ids ordered by (adapter, token id); tokens without adapter last
+ *   seg_start/len/adapter [min(T, n_adapters)]   runs of equal adapter, ascending adapter id
+ *   chunk_start/len/adapter [T]   each segment cut into pieces of <= group tokens, then the
+ *                       adapter-less tokens in pieces of <= group with adapter -1
+ *   counters [MLORA_CNT_WORDS]
+ * T <= MLORA_GATHER_MAX_T.  All outputs are exact integers / copied floats (bit-exact).
+ */
+int mlora_pool_gather(const int32_t *tok_adapter, int T,
+                      const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                      int n_adapters, int max_pages, int page_rows,
+                      int32_t *out_row_off, int32_t *out_rank, float *out_scale,
+                      int32_t *perm, int32_t *seg_start, int32_t *seg_len, int32_t *seg_adapter,
+                      int32_t *chunk_start, int32_t *chunk_len, int32_t *chunk_adapter, int group,
+                      int32_t *counters, void *stream);
+
+/*
+ * Decode (BGMV): for every token t with adapter a = tok_adapter[t] and every projection p
+ *     y_p[t] = (accumulate ? y_p[t] : 0) + scaling[a] * (x_p[t] . A_{p,a}) . B_{p,a}
+ * shrink and expand fused in one launch, rank-r intermediate kept on chip in fp32.
+ * Replaces punica.ops.add_lora_bgmv at lora_gpu.py:138,150,162 plus the
+ * `torch.zeros` before it (accumulate = 0) or the `q += q_lora` after it
+ * (transformer_layer_infer.py:160-171, accumulate = 1).
+ *
+ * y, x, a_rows, b_rows, hin, hout are HOST arrays of n_proj entries (device pointers /
+ * sizes per projection; projections may share x).  x_p is [T, hin[p]], y_p is [T, hout[p]].
+ * The page tables, rank and scaling are shared by all projections of the call.
+ * n_pages_a / n_pages_b bound the page ids (rows slab extents) for in-kernel checks.
+ * Grouped launch: pass the perm / chunk_* / counters arrays written by
+ * mlora_pool_gather with the same `group` (1, 2, 4 or 8) and max_chunks = T; tokens of one
+ * adapter then share one read of its rows.  With perm == NULL every token is its own
+ * work item and group must be 1.
+ */
+int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
+                     const void *const *a_rows, const void *const *b_rows,
+                     const int32_t *hin, const int32_t *hout,
+                     const int32_t *tok_adapter, int T,
+                     const int32_t *a_page_tbl, const int32_t *b_page_tbl,
+                     const int32_t *rank, const float *scaling,
+                     int n_adapters, int max_pages, int page_rows,
+                     int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+                     const int32_t *perm, const int32_t *chunk_start, const int32_t *chunk_len,
+                     const int32_t *chunk_adapter, const int32_t *counters, int group,
+                     int dtype, int accumulate, void *stream);
+
+/* One projection, one token per work item: the plain form of the call above. */
+int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
+               const int32_t *tok_adapter,
+               const int32_t *a_page_tbl, const int32_t *b_page_tbl,
+               const int32_t *rank, const float *scaling,
+               int T, int hin, int hout, int n_adapters, int max_pages, int page_rows,
+               int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               int dtype, int accumulate, void *stream);
+
+/*
+ * The reference's own layout and call, for drop-in and parity
+ * (lora_gpu.py:33-40 pool shapes, :137-138 call):
+ *   wa_T_all [N, L, r, hin], wb_T_all [N, L, hout, r] contiguous, indices int64 [T] in [0, N),
+ *   y[t] += scale * (x[t] . wa_T_all[idx[t], layer]^T) . wb_T_all[idx[t], layer]^T.
+ * An index outside [0, N) leaves that token's row untouched (the reference reads out of
+ * bounds there).
+ */
+int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const void *wb_T_all,
+                         const int64_t *indices, int T, int N, int L, int r, int hin, int hout,
+                         int layer_idx, float scale, int dtype, void *stream);
+
+/*
+ * Prefill (SGMV): tokens are packed contiguously per segment; segment s covers tokens
+ * [seg_start[s], seg_start[s] + seg_len[s]) and uses adapter seg_adapter[s] (negative = none):
+ *     y[t] = (accumulate ? y[t] : 0) + scaling[a] * (x[t] . A_a) . B_a
+ * computed on MFMA tiles with an fp32 [T, rank] intermediate that stays in `workspace`.
+ * Replaces torch.bmm(torch.bmm(x, A), B) at lora_gpu.py:127-128,145-146,157-158 without the
+ * per-call weight transposes/copies or the padding to equal prompt length.
+ * seg_* are device arrays of n_seg entries.  Segments must not overlap; tokens covered by no
+ * segment keep y (accumulate) or get zeros.  workspace: mlora_sgmv_workspace_bytes(T, n_seg).
+ */
+int64_t mlora_sgmv_workspace_bytes(int T, int n_seg);
+int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
+               const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+               const int32_t *a_page_tbl, const int32_t *b_page_tbl,
+               const int32_t *rank, const float *scaling,
+               int T, int hin, int hout, int n_adapters, int max_pages, int page_rows,
+               int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * The reference's prefill call on its own layout (lora_gpu.py:125-128): request b uses
+ * adapter slot b; x [B, Lpad, hin]; A_T [>=B, L, r, hin]; B_T [>=B, L, hout, r];
+ * y [B, Lpad, hout] = (x[b] . A_T[b, layer]^T) . B_T[b, layer]^T   (y is overwritten).
+ */
+int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void *B_T,
+                            int B, int Lpad, int L, int r, int hin, int hout, int layer_idx,
+                            int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLORA_H */

@@ -1,0 +1,481 @@
+/*
+ * mlora_oracle.c -- CPU restatement of the multi-LoRA batched-apply path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the checker the HIP kernels are
+ * compared against; it is never linked into, imported by, or called from the
+ * shipped library or its Python host layer.  Only tests, the smoke check and
+ * the benchmark's cpu_baseline leg load it.
+ *
+ * Every function restates, in plain scalar C, what the reference computes on
+ * this path.  The reference's decode arithmetic lives in a third-party module
+ * (punica==0.2.0, requirements.txt:75) that is not in the reference tree, so
+ * that call is restated from its call sites and documented contract
+ * (lightllm/models/lora_gpu.py:138,150,162:
+ *     y[i] += x[i] @ wa_T_all[idx[i], layer].T @ wb_T_all[idx[i], layer].T * scale)
+ * -- parity against punica's own outputs is UNPINNED (no vectors exist); what
+ * is pinned, by the tests under tests/, is this file against closed forms,
+ * brute force, library matmuls and invariants.
+ *
+ * Pinned functions (see tests/test_oracle_*.py):
+ *   orc_f16_to_f32 / orc_f32_to_f16 / orc_bf16_* : exhaustive / randomized vs numpy & torch
+ *   orc_pool_gather, orc_build_segments, orc_build_chunks, orc_sgmv_plan : vs numpy closed forms
+ *   orc_lora_apply_paged      : brute-force fp64 loops, one-hot, scale 0, library matmul
+ *   orc_add_lora_bgmv_ref     : same expression through numpy on the reference layout
+ *   orc_prefill_bmm_ref       : numpy matmul pairs (the reference's bmm.bmm)
+ *   orc_cpu_lora_worker       : numpy fp32 matmul of the reference's one-line arithmetic
+ *   orc_cpu_chunk_plan        : enumeration of the reference's chunk index arithmetic
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <string.h>
+#include <stdlib.h>
+#include <math.h>
+#include <pthread.h>
+
+#define ORC_OK 0
+#define ORC_EINVAL (-1)
+#define ORC_ERANGE (-2)
+
+/* ------------------------------------------------------------------ */
+/* 16-bit float conversions (IEEE binary16 and bfloat16), RNE.         */
+/* ------------------------------------------------------------------ */
+
+static inline uint32_t f32_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float bits_f32(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+
+float orc_f16_to_f32(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (exp == 0) {
+        if (man == 0) return bits_f32(sign);
+        /* subnormal: value = man * 2^-24 */
+        float v = (float)man * 5.9604644775390625e-08f;
+        return sign ? -v : v;
+    }
+    if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+    return bits_f32(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t orc_f32_to_f16(float f)
+{
+    uint32_t u = f32_bits(f);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t a = u & 0x7fffffffu;
+    if (a >= 0x7f800000u) {                    /* inf / nan */
+        if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x3ffu));
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (a >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);   /* rounds to >= 65520 -> inf */
+    if (a < 0x33000001u) return sign;          /* below half of the smallest subnormal */
+    int32_t e = (int32_t)(a >> 23) - 127;
+    uint32_t m = (a & 0x7fffffu) | 0x800000u;  /* 24-bit significand */
+    int shift;
+    uint32_t base;
+    if (e < -14) { shift = 13 + (-14 - e); base = 0; }          /* subnormal result */
+    else { shift = 13; base = (uint32_t)(e + 15) << 10; m &= 0x7fffffu; }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | (base + q));      /* carry into the exponent is correct by construction */
+}
+
+float orc_bf16_to_f32(uint16_t b) { return bits_f32((uint32_t)b << 16); }
+
+uint16_t orc_f32_to_bf16(float f)
+{
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  /* quiet nan */
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7fffu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+static inline float ld16(const uint16_t *p, size_t i, int dtype)
+{
+    return dtype == 0 ? orc_f16_to_f32(p[i]) : orc_bf16_to_f32(p[i]);
+}
+static inline uint16_t st16(float v, int dtype)
+{
+    return dtype == 0 ? orc_f32_to_f16(v) : orc_f32_to_bf16(v);
+}
+
+/* vector helpers so that tests can pin the conversions wholesale */
+void orc_f16_to_f32_n(const uint16_t *in, float *out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_f16_to_f32(in[i]); }
+void orc_f32_to_f16_n(const float *in, uint16_t *out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_f32_to_f16(in[i]); }
+void orc_bf16_to_f32_n(const uint16_t *in, float *out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_bf16_to_f32(in[i]); }
+void orc_f32_to_bf16_n(const float *in, uint16_t *out, size_t n) { for (size_t i = 0; i < n; i++) out[i] = orc_f32_to_bf16(in[i]); }
+
+/* ------------------------------------------------------------------ */
+/* Adapter-pool index / offset gather.                                 */
+/* The reference keeps a dense pool indexed [adapter, layer, ...]       */
+/* (lightllm/models/lora_gpu.py:33-40) and a per-token index vector     */
+/* (lora_gpu.py:120,124).  The paged pool generalises that: rank row j  */
+/* of adapter i lives at row  page_tbl[i][j / page_rows] * page_rows    */
+/* + j % page_rows.  Out-of-range adapters are an error here (the       */
+/* reference would read out of bounds, lora_gpu.py:120 vs manager.py:88)*/
+/* and a negative adapter means "no adapter for this token".           */
+/* ------------------------------------------------------------------ */
+
+int orc_pool_gather(const int32_t *tok_adapter, int T,
+                    const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                    int n_adapters, int max_pages, int page_rows,
+                    int32_t *out_row_off /* [T, max_pages] */, int32_t *out_rank /* [T] */,
+                    float *out_scale /* [T] */)
+{
+    if (T < 0 || n_adapters < 0 || max_pages <= 0 || page_rows <= 0) return ORC_EINVAL;
+    for (int t = 0; t < T; t++) {
+        int a = tok_adapter[t];
+        if (a >= n_adapters) return ORC_ERANGE;
+        if (a < 0) {
+            out_rank[t] = 0;
+            out_scale[t] = 0.0f;
+            for (int p = 0; p < max_pages; p++) out_row_off[(size_t)t * max_pages + p] = -1;
+            continue;
+        }
+        int r = rank[a];
+        int np = (r + page_rows - 1) / page_rows;
+        if (np > max_pages) return ORC_ERANGE;
+        out_rank[t] = r;
+        out_scale[t] = scaling[a];
+        for (int p = 0; p < max_pages; p++)
+            out_row_off[(size_t)t * max_pages + p] = p < np ? page_tbl[(size_t)a * max_pages + p] * page_rows : -1;
+    }
+    return ORC_OK;
+}
+
+/* Stable grouping of tokens by adapter: perm lists token ids ordered by
+ * (adapter, token id); tokens with a negative adapter come last and belong to
+ * no segment.  Segments are runs of equal adapter in that order, ascending in
+ * adapter id.  Returns the number of tokens that have an adapter in *n_valid. */
+int orc_build_segments(const int32_t *tok_adapter, int T, int n_adapters,
+                       int32_t *perm /* [T] */, int32_t *seg_start, int32_t *seg_len,
+                       int32_t *seg_adapter /* each [min(T, n_adapters)] */,
+                       int32_t *n_seg, int32_t *n_valid)
+{
+    if (T < 0 || n_adapters < 0) return ORC_EINVAL;
+    int32_t *count = (int32_t *)calloc((size_t)n_adapters + 1, sizeof(int32_t));
+    int32_t *start = (int32_t *)calloc((size_t)n_adapters + 1, sizeof(int32_t));
+    if (!count || !start) { free(count); free(start); return ORC_EINVAL; }
+    int valid = 0;
+    for (int t = 0; t < T; t++) {
+        int a = tok_adapter[t];
+        if (a >= n_adapters) { free(count); free(start); return ORC_ERANGE; }
+        if (a >= 0) { count[a]++; valid++; }
+    }
+    int ns = 0, pos = 0;
+    for (int a = 0; a < n_adapters; a++) {
+        start[a] = pos;
+        if (count[a] > 0) {
+            seg_start[ns] = pos; seg_len[ns] = count[a]; seg_adapter[ns] = a; ns++;
+        }
+        pos += count[a];
+    }
+    int tail = valid;
+    for (int t = 0; t < T; t++) {                 /* ascending t => stable */
+        int a = tok_adapter[t];
+        if (a >= 0) perm[start[a]++] = t; else perm[tail++] = t;
+    }
+    *n_seg = ns; *n_valid = valid;
+    free(count); free(start);
+    return ORC_OK;
+}
+
+/* Decode work list: every segment is cut into chunks of at most `group`
+ * tokens; chunk c covers sorted positions [chunk_start[c], chunk_start[c] +
+ * chunk_len[c]) and uses chunk_adapter[c].  Tokens without an adapter form
+ * trailing chunks with adapter -1 (they only matter when the caller asks for
+ * y = delta, where their rows must be written as zero). */
+int orc_build_chunks(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter,
+                     int n_seg, int n_valid, int T, int group,
+                     int32_t *chunk_start, int32_t *chunk_len, int32_t *chunk_adapter, int32_t *n_chunks)
+{
+    if (group <= 0) return ORC_EINVAL;
+    int nc = 0;
+    for (int s = 0; s < n_seg; s++)
+        for (int o = 0; o < seg_len[s]; o += group) {
+            chunk_start[nc] = seg_start[s] + o;
+            chunk_len[nc] = seg_len[s] - o < group ? seg_len[s] - o : group;
+            chunk_adapter[nc] = seg_adapter[s];
+            nc++;
+        }
+    for (int o = n_valid; o < T; o += group) {
+        chunk_start[nc] = o;
+        chunk_len[nc] = T - o < group ? T - o : group;
+        chunk_adapter[nc] = -1;
+        nc++;
+    }
+    *n_chunks = nc;
+    return ORC_OK;
+}
+
+/* Prefill work list: every segment (a request's contiguous tokens, as the
+ * reference batches one adapter slot per request, lora_gpu.py:125-128) is cut
+ * into tiles of `tile` tokens.  tile_seg / tile_tok0 / tile_ntok per tile. */
+int orc_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, int n_seg, int tile,
+                  int32_t *tile_seg, int32_t *tile_tok0, int32_t *tile_ntok, int32_t *n_tiles)
+{
+    if (tile <= 0) return ORC_EINVAL;
+    int nt = 0;
+    for (int s = 0; s < n_seg; s++)
+        for (int o = 0; o < seg_len[s]; o += tile) {
+            tile_seg[nt] = s;
+            tile_tok0[nt] = seg_start[s] + o;
+            tile_ntok[nt] = seg_len[s] - o < tile ? seg_len[s] - o : tile;
+            nt++;
+        }
+    *n_tiles = nt;
+    return ORC_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* LoRA apply over the paged pool:                                     */
+/*   y[t] = round16( y0[t] + s_a * (x[t] . A_a) . B_a ),  a = adapter   */
+/* A rows are rank rows of length Hin (A^T), B rows are rank rows of    */
+/* length Hout; accumulation in fp32 (acc64 = 0) or fp64 (acc64 = 1),   */
+/* one rounding to the 16-bit type at the end.  The reference rounds    */
+/* the delta first and adds in fp16 (lora_gpu.py:137-138 then           */
+/* transformer_layer_infer.py:160-171); single rounding is the stated   */
+/* contract of this build and differs by at most one ulp of y.          */
+/* y0 == NULL means y = delta.                                         */
+/* ------------------------------------------------------------------ */
+
+int orc_lora_apply_paged(uint16_t *y, const uint16_t *y0, const uint16_t *x,
+                         const uint16_t *a_rows, const uint16_t *b_rows,
+                         const int32_t *tok_adapter,
+                         const int32_t *a_page_tbl, const int32_t *b_page_tbl,
+                         const int32_t *rank, const float *scaling,
+                         int T, int Hin, int Hout, int n_adapters, int max_pages, int page_rows,
+                         int dtype, int acc64)
+{
+    if (T < 0 || Hin <= 0 || Hout <= 0 || max_pages <= 0 || page_rows <= 0) return ORC_EINVAL;
+    if (dtype != 0 && dtype != 1) return ORC_EINVAL;
+    for (int t = 0; t < T; t++) {
+        int a = tok_adapter[t];
+        if (a >= n_adapters) return ORC_ERANGE;
+        if (a >= 0 && (rank[a] + page_rows - 1) / page_rows > max_pages) return ORC_ERANGE;
+    }
+    double *vd = (double *)malloc(sizeof(double) * (size_t)max_pages * page_rows);
+    float *vf = (float *)malloc(sizeof(float) * (size_t)max_pages * page_rows);
+    if (!vd || !vf) { free(vd); free(vf); return ORC_EINVAL; }
+    for (int t = 0; t < T; t++) {
+        int a = tok_adapter[t];
+        const uint16_t *xt = x + (size_t)t * Hin;
+        uint16_t *yt = y + (size_t)t * Hout;
+        if (a < 0) {
+            for (int c = 0; c < Hout; c++) yt[c] = y0 ? y0[(size_t)t * Hout + c] : 0;
+            continue;
+        }
+        int r = rank[a];
+        float s = scaling[a];
+        for (int j = 0; j < r; j++) {
+            size_t row = (size_t)a_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+            const uint16_t *ar = a_rows + row * Hin;
+            if (acc64) {
+                double acc = 0.0;
+                for (int k = 0; k < Hin; k++) acc += (double)ld16(xt, k, dtype) * (double)ld16(ar, k, dtype);
+                vd[j] = acc;
+            } else {
+                float acc = 0.0f;
+                for (int k = 0; k < Hin; k++) acc += ld16(xt, k, dtype) * ld16(ar, k, dtype);
+                vf[j] = acc;
+            }
+        }
+        for (int c = 0; c < Hout; c++) {
+            if (acc64) {
+                double acc = 0.0;
+                for (int j = 0; j < r; j++) {
+                    size_t row = (size_t)b_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+                    acc += vd[j] * (double)ld16(b_rows + row * Hout, c, dtype);
+                }
+                double base = y0 ? (double)ld16(y0 + (size_t)t * Hout, c, dtype) : 0.0;
+                yt[c] = st16((float)(base + (double)s * acc), dtype);
+            } else {
+                float acc = 0.0f;
+                for (int j = 0; j < r; j++) {
+                    size_t row = (size_t)b_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+                    acc += vf[j] * ld16(b_rows + row * Hout, c, dtype);
+                }
+                float base = y0 ? ld16(y0 + (size_t)t * Hout, c, dtype) : 0.0f;
+                yt[c] = st16(base + s * acc, dtype);
+            }
+        }
+    }
+    free(vd); free(vf);
+    return ORC_OK;
+}
+
+/* The reference's decode call on the reference's own layout
+ * (lora_gpu.py:33-40,137-138): wa_T_all [N, L, r, Hin], wb_T_all [N, L, Hout, r],
+ * fp16, indices int64 [T];  y[t] += scale * (x[t] . wa[idx,layer]^T) . wb[idx,layer]^T. */
+int orc_add_lora_bgmv_ref(uint16_t *y, const uint16_t *x,
+                          const uint16_t *wa_T_all, const uint16_t *wb_T_all,
+                          const int64_t *indices, int T, int N, int L, int r,
+                          int Hin, int Hout, int layer_idx, float scale, int dtype)
+{
+    if (layer_idx < 0 || layer_idx >= L || r <= 0) return ORC_EINVAL;
+    float *v = (float *)malloc(sizeof(float) * (size_t)r);
+    if (!v) return ORC_EINVAL;
+    for (int t = 0; t < T; t++) {
+        int64_t a = indices[t];
+        if (a < 0 || a >= N) { free(v); return ORC_ERANGE; }
+        const uint16_t *wa = wa_T_all + ((size_t)a * L + layer_idx) * (size_t)r * Hin;
+        const uint16_t *wb = wb_T_all + ((size_t)a * L + layer_idx) * (size_t)Hout * r;
+        for (int j = 0; j < r; j++) {
+            float acc = 0.0f;
+            for (int k = 0; k < Hin; k++) acc += ld16(x + (size_t)t * Hin, k, dtype) * ld16(wa + (size_t)j * Hin, k, dtype);
+            v[j] = acc;
+        }
+        for (int c = 0; c < Hout; c++) {
+            float acc = 0.0f;
+            for (int j = 0; j < r; j++) acc += v[j] * ld16(wb + (size_t)c * r, j, dtype);
+            size_t o = (size_t)t * Hout + c;
+            y[o] = st16(ld16(y, o, dtype) + scale * acc, dtype);
+        }
+    }
+    free(v);
+    return ORC_OK;
+}
+
+/* The reference's prefill call (lora_gpu.py:125-128): request b uses adapter
+ * slot b; x [B, Lpad, Hin]; A_T [B, L, r, Hin]; B_T [B, L, Hout, r];
+ * y = bmm(bmm(x, A), B).  torch.bmm on fp16 stores its result in fp16, so the
+ * reference rounds the [B, Lpad, r] intermediate; round_mid = 1 restates that,
+ * round_mid = 0 keeps it in fp32 (this build's contract). */
+int orc_prefill_bmm_ref(uint16_t *y, const uint16_t *x, const uint16_t *A_T, const uint16_t *B_T,
+                        int Bsz, int Lpad, int L, int r, int Hin, int Hout, int layer_idx,
+                        int dtype, int round_mid)
+{
+    if (layer_idx < 0 || layer_idx >= L || r <= 0) return ORC_EINVAL;
+    float *v = (float *)malloc(sizeof(float) * (size_t)r);
+    if (!v) return ORC_EINVAL;
+    for (int b = 0; b < Bsz; b++) {
+        const uint16_t *wa = A_T + ((size_t)b * L + layer_idx) * (size_t)r * Hin;
+        const uint16_t *wb = B_T + ((size_t)b * L + layer_idx) * (size_t)Hout * r;
+        for (int l = 0; l < Lpad; l++) {
+            const uint16_t *xt = x + ((size_t)b * Lpad + l) * Hin;
+            for (int j = 0; j < r; j++) {
+                float acc = 0.0f;
+                for (int k = 0; k < Hin; k++) acc += ld16(xt, k, dtype) * ld16(wa + (size_t)j * Hin, k, dtype);
+                v[j] = round_mid ? ld16((uint16_t[]){st16(acc, dtype)}, 0, dtype) : acc;
+            }
+            for (int c = 0; c < Hout; c++) {
+                float acc = 0.0f;
+                for (int j = 0; j < r; j++) acc += v[j] * ld16(wb + (size_t)c * r, j, dtype);
+                y[((size_t)b * Lpad + l) * Hout + c] = st16(acc, dtype);
+            }
+        }
+    }
+    free(v);
+    return ORC_OK;
+}
+
+/* ------------------------------------------------------------------ */
+/* The CPU-assisted path's arithmetic (lora_cpu/lora_shm_op/app.py:     */
+/* 133-141): one worker takes a chunk of at most `cap` tokens of one    */
+/* request and one projection and computes                              */
+/*     res = x.float() @ down @ up ;  out = res.half()                  */
+/* with fp32 weights down [Hin, r], up [r, Hout] (app.py:38-45).        */
+/* ------------------------------------------------------------------ */
+
+int orc_cpu_lora_worker(const uint16_t *x /* [n_tok, Hin] fp16 */, const float *down, const float *up,
+                        uint16_t *out /* [n_tok, Hout] fp16 */, int n_tok, int Hin, int Hout, int r)
+{
+    if (n_tok < 0 || r <= 0) return ORC_EINVAL;
+    float *tmp = (float *)malloc(sizeof(float) * (size_t)r);
+    float *row = (float *)malloc(sizeof(float) * (size_t)Hout);
+    if (!tmp || !row) { free(tmp); free(row); return ORC_EINVAL; }
+    for (int t = 0; t < n_tok; t++) {
+        for (int j = 0; j < r; j++) tmp[j] = 0.0f;
+        for (int k = 0; k < Hin; k++) {
+            float xv = orc_f16_to_f32(x[(size_t)t * Hin + k]);
+            const float *d = down + (size_t)k * r;
+            for (int j = 0; j < r; j++) tmp[j] += xv * d[j];
+        }
+        for (int c = 0; c < Hout; c++) row[c] = 0.0f;
+        for (int j = 0; j < r; j++) {
+            const float *u = up + (size_t)j * Hout;
+            float tv = tmp[j];
+            for (int c = 0; c < Hout; c++) row[c] += tv * u[c];
+        }
+        for (int c = 0; c < Hout; c++) out[(size_t)t * Hout + c] = orc_f32_to_f16(row[c]);
+    }
+    free(tmp); free(row);
+    return ORC_OK;
+}
+
+/* Chunk arithmetic of the CPU-assisted path.  The driver cuts each request's
+ * tkn_num tokens into cpu_per_request = (tkn_num-1)/cap + 1 chunks
+ * (lightllm/models/lora_cpu.py:150-151); worker `row_id` serves request
+ * dim_0 = row_id / cpu_per_request, chunk dim_1 = row_id % cpu_per_request,
+ * tokens [dim_1*cap, min((dim_1+1)*cap, tkn_num)) (app.py:133-136, restated
+ * from the math: the reference clips tkn_num to cap before the worker sees it,
+ * lora_cpu.py:175, which only agrees with this when a request fits one chunk).
+ * The collector places chunk (b, dim_1) at token offset dim_1*cap of request b,
+ * last chunk holding tkn_num - (cpr-1)*cap tokens (lora_cpu.py:210-232). */
+int orc_cpu_chunk_plan(int batch, int tkn_num, int cap,
+                       int32_t *req /* [batch*cpr] */, int32_t *tok0, int32_t *ntok, int32_t *n_chunks)
+{
+    if (batch < 0 || tkn_num <= 0 || cap <= 0) return ORC_EINVAL;
+    int cpr = (tkn_num - 1) / cap + 1;
+    int n = 0;
+    for (int row_id = 0; row_id < batch * cpr; row_id++) {
+        int d0 = row_id / cpr, d1 = row_id % cpr;
+        int end = (d1 + 1) * cap < tkn_num ? (d1 + 1) * cap : tkn_num;
+        req[n] = d0; tok0[n] = d1 * cap; ntok[n] = end - d1 * cap; n++;
+    }
+    *n_chunks = n;
+    return ORC_OK;
+}
+
+/* Whole CPU-assisted LoRA delta for one projection over a batch of equal-length
+ * requests, sharded as the reference shards it: one task per (request, chunk),
+ * tasks spread over n_threads pinned-worker stand-ins.  Request b uses adapter
+ * req_adapter[b] of the fp32 weight sets down[N][Hin][r], up[N][r][Hout].
+ * Used for the benchmark's cpu_baseline leg and checked against
+ * orc_cpu_lora_worker applied chunk by chunk. */
+typedef struct {
+    const uint16_t *x; const float *down; const float *up; uint16_t *out;
+    const int32_t *req_adapter; const int32_t *req; const int32_t *tok0; const int32_t *ntok;
+    int n_chunks, tkn_num, Hin, Hout, r, tid, n_threads;
+} orc_cpu_job;
+
+static void *orc_cpu_thread(void *arg)
+{
+    orc_cpu_job *j = (orc_cpu_job *)arg;
+    for (int c = j->tid; c < j->n_chunks; c += j->n_threads) {
+        int b = j->req[c];
+        size_t tok = (size_t)b * j->tkn_num + j->tok0[c];
+        int a = j->req_adapter[b];
+        orc_cpu_lora_worker(j->x + tok * j->Hin,
+                            j->down + (size_t)a * j->Hin * j->r, j->up + (size_t)a * j->r * j->Hout,
+                            j->out + tok * j->Hout, j->ntok[c], j->Hin, j->Hout, j->r);
+    }
+    return NULL;
+}
+
+int orc_cpu_lora_batch(const uint16_t *x, const float *down, const float *up, uint16_t *out,
+                       const int32_t *req_adapter, int batch, int tkn_num, int cap,
+                       int Hin, int Hout, int r, int n_threads)
+{
+    if (n_threads <= 0 || n_threads > 256) return ORC_EINVAL;
+    int cpr = (tkn_num - 1) / cap + 1;
+    int32_t *req = (int32_t *)malloc(sizeof(int32_t) * 3 * (size_t)batch * cpr);
+    if (!req) return ORC_EINVAL;
+    int32_t *tok0 = req + (size_t)batch * cpr, *ntok = tok0 + (size_t)batch * cpr;
+    int32_t nc = 0;
+    int rc = orc_cpu_chunk_plan(batch, tkn_num, cap, req, tok0, ntok, &nc);
+    if (rc) { free(req); return rc; }
+    orc_cpu_job jobs[256];
+    pthread_t th[256];
+    for (int i = 0; i < n_threads; i++) {
+        jobs[i] = (orc_cpu_job){x, down, up, out, req_adapter, req, tok0, ntok, nc, tkn_num, Hin, Hout, r, i, n_threads};
+        if (i > 0) pthread_create(&th[i], NULL, orc_cpu_thread, &jobs[i]);
+    }
+    orc_cpu_thread(&jobs[0]);
+    for (int i = 1; i < n_threads; i++) pthread_join(th[i], NULL);
+    free(req);
+    return ORC_OK;
+}

@@ -1,0 +1,81 @@
+"""CPU-side checks of the C ABI: the library loads, exports every function include/mlora.h declares
+with the arity the Python binding uses, and rejects bad arguments before touching the GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from mlora import _ext
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mlora.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:const\s+char\s*\*|int64_t|int)\s*(mlora_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args == "void" else len([a for a in args.split(",") if a.strip()])
+    return out
+
+
+def test_header_and_binding_agree():
+    decl = _declared()
+    assert set(decl) == set(_ext.SIGNATURES), (sorted(decl), sorted(_ext.SIGNATURES))
+    for name, n in decl.items():
+        assert len(_ext.SIGNATURES[name][1]) == n, name
+
+
+def test_library_exports_every_symbol():
+    lib = _ext.lib()
+    for name in _declared():
+        assert hasattr(lib, name), name
+    assert lib.mlora_version() >= 100
+
+
+def test_validation_errors_without_gpu():
+    lib = _ext.lib()
+    one = C.c_void_p(16)      # never dereferenced: every call below fails validation first
+    P = (C.c_void_p * 8)(16, 16, 16, 16, 16, 16, 16, 16)
+    H = (C.c_int32 * 8)(64, 64, 64, 64, 64, 64, 64, 64)
+
+    def bgmv(**kw):
+        a = dict(n_proj=1, hin=H, T=4, n_adapters=4, max_pages=8, page_rows=8, npa=10, npb=10, max_rank=64, perm=None,
+                 group=1, dtype=0, y=P)
+        a.update(kw)
+        return lib.mlora_bgmv_multi(a["n_proj"], a["y"], P, P, P, a["hin"], H, one, a["T"], one, one, one, one,
+                                    a["n_adapters"], a["max_pages"], a["page_rows"], a["npa"], a["npb"], a["max_rank"],
+                                    a["perm"], None, None, None, None, a["group"], a["dtype"], 1, None)
+
+    assert bgmv(T=0) == _ext.MLORA_OK
+    assert bgmv(dtype=7) == _ext.MLORA_EDTYPE
+    assert b"dtype" in lib.mlora_last_error()
+    assert bgmv(n_proj=9) == _ext.MLORA_ERANGE
+    assert bgmv(max_rank=65) == _ext.MLORA_ERANGE
+    assert bgmv(page_rows=3) == _ext.MLORA_EINVAL
+    assert bgmv(max_pages=1, page_rows=8, max_rank=16) == _ext.MLORA_ERANGE
+    assert bgmv(hin=(C.c_int32 * 8)(60, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
+    assert bgmv(y=(C.c_void_p * 8)(8, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
+    assert bgmv(group=4) == _ext.MLORA_EINVAL          # grouped launch without the grouped view
+    assert bgmv(T=-1) == _ext.MLORA_EINVAL
+    with pytest.raises(_ext.MloraError) as e:
+        _ext.check(bgmv(dtype=7))
+    assert e.value.code == _ext.MLORA_EDTYPE
+
+    rc = lib.mlora_pool_gather(one, 9000, one, one, one, 4, 8, 8, None, None, None, one, one, one, one, one, one, one, 4, one, None)
+    assert rc == _ext.MLORA_ERANGE                     # more tokens than one gather call groups
+    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, None, None, None, one, None, one, one, one, one, one, 4, one, None)
+    assert rc == _ext.MLORA_EINVAL                     # incomplete grouped view
+    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, None, None, None, one, one, one, one, one, one, one, 3, one, None)
+    assert rc == _ext.MLORA_EINVAL                     # group not a power of two
+
+    assert lib.mlora_sgmv_workspace_bytes(9089, 16) > 9089 * 64 * 4
+    rc = lib.mlora_sgmv(one, one, one, one, one, one, one, 2, one, one, one, one, 100, 64, 64, 4, 8, 8, 10, 10, 64, 1, 1,
+                        one, 16, None)
+    assert rc == _ext.MLORA_ENOSPACE
+    rc = lib.mlora_bgmv_reflayout(one, one, one, one, one, 4, 8, 32, 16, 64, 64, 32, 1.0, 0, None)
+    assert rc == _ext.MLORA_ERANGE                     # layer_idx == L
+    rc = lib.mlora_prefill_reflayout(one, one, one, one, 2, 16, 4, 12, 64, 64, 0, 0, one, 1 << 30, None)
+    assert rc == _ext.MLORA_ERANGE                     # rank not a multiple of 8

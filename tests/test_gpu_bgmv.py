@@ -1,0 +1,199 @@
+"""GPU parity: fused BGMV decode kernel through the C ABI against the fp32-accumulated oracle
+(rtol 1e-2 / atol 1e-3), on seeded inputs, plus size-independent properties at full size."""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import (ATOL, RTOL, assert_close_bits, oracle_apply, say, tdtype, upload_pool)
+from helpers import BF16, FP16, PagedPool, bits_of, bits_to_torch, f32_of, torch_to_bits
+from mlora import bgmv, lora_apply, plan_decode
+
+pytestmark = pytest.mark.gpu
+
+
+def _zipf(rng, T, N, alpha):
+    p = np.arange(1, N + 1, dtype=np.float64) ** -alpha
+    return rng.permutation(N)[rng.choice(N, size=T, p=p / p.sum())].astype(np.int32)
+
+
+def _run(pp, x_bits, tok, y0_bits, group, accumulate=True):
+    pool = upload_pool(pp)
+    x = bits_to_torch(x_bits, pp.dtype, "cuda")
+    y = bits_to_torch(y0_bits, pp.dtype, "cuda") if y0_bits is not None else \
+        torch.full((len(tok), pp.hout), float("nan"), dtype=tdtype(pp.dtype), device="cuda")
+    t = torch.from_numpy(tok).cuda()
+    plan = plan_decode(t, pool, group=group) if group > 0 else None
+    bgmv([y], [x], pool, 0, ["p"], t, plan=plan, accumulate=accumulate)
+    torch.cuda.synchronize()
+    return torch_to_bits(y)
+
+
+CASES = [
+    # name, T, ranks, hin, hout, alpha, dtype
+    ("C1 q_proj T=32 8xr16", 32, [16] * 8, 4096, 4096, 0.0, FP16),
+    ("C2 q_proj T=256 64xr16 zipf1.0", 256, [16] * 64, 4096, 4096, 1.0, FP16),
+    ("C2 bf16", 256, [16] * 64, 4096, 4096, 1.0, BF16),
+    ("C3 hetero 4096x4096", 128, None, 4096, 4096, 1.2, FP16),
+    ("C3 hetero gate 4096x11008", 128, None, 4096, 11008, 1.2, FP16),
+    ("C3 hetero down 11008x4096", 128, None, 11008, 4096, 1.2, FP16),
+    ("C5 slice T=512 r32", 512, [32] * 200, 4096, 4096, 1.1, FP16),
+    ("odd widths 200x72", 19, [8, 24, 5, 64, 1], 200, 72, 0.5, BF16),
+]
+
+
+_CASE_CACHE = {}
+
+
+def _case(name):
+    """Seeded inputs and oracle outputs of one case (computed once, shared by the launch variants)."""
+    if name not in _CASE_CACHE:
+        _, T, ranks, hin, hout, alpha, dtype = next(c for c in CASES if c[0] == name)
+        rng = np.random.default_rng(zlib.crc32(name.encode()))
+        if ranks is None:
+            ranks = rng.choice([8, 16, 32, 64], 128)
+        N = len(ranks)
+        pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=dtype)
+        tok = _zipf(rng, T, N, alpha) if alpha > 0 else rng.integers(0, N, T).astype(np.int32)
+        x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype)
+        y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), dtype)
+        _CASE_CACHE[name] = (pp, tok, x, y0, oracle_apply(pp, x, tok, y0), oracle_apply(pp, x, tok, None))
+    return _CASE_CACHE[name]
+
+
+@pytest.mark.parametrize("name", [c[0] for c in CASES])
+@pytest.mark.parametrize("group", [0, 1, 4])
+def test_bgmv_vs_oracle(name, group):
+    dtype = next(c for c in CASES if c[0] == name)[6]
+    pp, tok, x, y0, want, want_d = _case(name)
+    say(f"bgmv {name} group={group} accumulate")
+    got = _run(pp, x, tok, y0, group)
+    assert_close_bits(got, want, dtype, name)
+    # the delta alone must also meet the tolerance (y = delta form, reference's zeros+bgmv at lora_gpu.py:137-138)
+    say(f"bgmv {name} group={group} delta")
+    got_d = _run(pp, x, tok, None, group, accumulate=False)
+    assert_close_bits(got_d, want_d, dtype, name + " delta")
+
+
+@pytest.mark.parametrize("group", [0, 2, 8])
+def test_bgmv_integer_inputs_bit_exact(group):
+    """Integer-valued inputs make every fp32 operation exact: the kernel must match bit for bit."""
+    rng = np.random.default_rng(41)
+    ranks = [8, 16, 3, 1, 5, 32]
+    pp = PagedPool(rng, ranks, hin=512, hout=256, page_rows=8, dtype=FP16, integer=True)
+    pp.scaling[:] = [1, 2, 0.5, -1, 4, 0.25]
+    T = 61
+    tok = rng.integers(-1, len(ranks), T).astype(np.int32)
+    # sparse integer activations keep |sums| < 2048 (exact in fp16)
+    xi = (rng.integers(-2, 3, (T, 512)) * (rng.random((T, 512)) < 0.06)).astype(np.float32)
+    y0 = bits_of(rng.integers(-8, 9, (T, 256)).astype(np.float32), FP16)
+    x = bits_of(xi, FP16)
+    want = oracle_apply(pp, x, tok, y0)
+    assert np.abs(f32_of(want, FP16)).max() < 2048
+    say(f"bgmv integer-valued inputs group={group}")
+    got = _run(pp, x, tok, y0, group)
+    assert np.array_equal(got, want)
+
+
+def test_bgmv_tokens_without_adapter_and_rank_tails():
+    rng = np.random.default_rng(42)
+    pp = PagedPool(rng, [7, 9, 33, 64, 2], 1024, 1024, page_rows=8, dtype=FP16)
+    T = 40
+    tok = rng.integers(-1, 5, T).astype(np.int32)
+    tok[:3] = -1
+    x = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
+    y0 = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
+    for group in (0, 4):
+        say(f"bgmv no-adapter tokens group={group}")
+        got = _run(pp, x, tok, y0, group)
+        assert np.array_equal(got[tok < 0], y0[tok < 0])          # untouched, bit for bit
+        assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16)
+        got_d = _run(pp, x, tok, None, group, accumulate=False)
+        assert np.all(got_d[tok < 0] == 0)                        # y = delta defines those rows as zero
+        assert_close_bits(got_d, oracle_apply(pp, x, tok, None), FP16)
+
+
+def test_bgmv_multi_projection_one_launch():
+    """q/k/v share x, o has its own input: one launch, four slabs, each checked against the oracle."""
+    rng = np.random.default_rng(43)
+    T, N, H = 96, 24, 1024
+    ranks = rng.choice([8, 16, 32], N)
+    pps = {p: PagedPool(np.random.default_rng(50), ranks, H, H, page_rows=8, dtype=FP16) for p in "qkvo"}
+    for i, p in enumerate("qkvo"):      # same page table, different weights per projection
+        r2 = np.random.default_rng(60 + i)
+        pps[p].a_rows = bits_of((r2.standard_normal(pps[p].a_rows.shape) * 0.02).astype(np.float32), FP16)
+        pps[p].b_rows = bits_of((r2.standard_normal(pps[p].b_rows.shape) * 0.02).astype(np.float32), FP16)
+    pool = upload_pool(pps["q"], projections={p: (H, H) for p in "qkvo"})
+    for p in "qkvo":
+        pool.a_rows[p][0].copy_(bits_to_torch(pps[p].a_rows, FP16))
+        pool.b_rows[p][0].copy_(bits_to_torch(pps[p].b_rows, FP16))
+    tok = _zipf(rng, T, N, 1.0)
+    x_qkv = bits_of(rng.standard_normal((T, H)).astype(np.float32), FP16)
+    x_o = bits_of(rng.standard_normal((T, H)).astype(np.float32), FP16)
+    y0 = {p: bits_of(rng.standard_normal((T, H)).astype(np.float32), FP16) for p in "qkvo"}
+    t = torch.from_numpy(tok).cuda()
+    xs = {p: bits_to_torch(x_o if p == "o" else x_qkv, FP16, "cuda") for p in "qkvo"}
+    ys = {p: bits_to_torch(y0[p], FP16, "cuda") for p in "qkvo"}
+    plan = plan_decode(t, pool, group=4)
+    say("bgmv 4 projections in one launch")
+    bgmv([ys[p] for p in "qkvo"], [xs[p] for p in "qkvo"], pool, 0, list("qkvo"), t, plan=plan)
+    torch.cuda.synchronize()
+    for p in "qkvo":
+        want = oracle_apply(pps[p], x_o if p == "o" else x_qkv, tok, y0[p])
+        assert_close_bits(torch_to_bits(ys[p]), want, FP16, f"projection {p}")
+
+
+def test_bgmv_full_size_properties():
+    """Config-2 size, no oracle: permutation equivariance, page-placement invariance, grouped == ungrouped
+    within tolerance, linearity of the delta, and lora_apply == bgmv."""
+    rng = np.random.default_rng(44)
+    T, N, H = 256, 64, 4096
+    pp = PagedPool(rng, [16] * N, H, H, page_rows=8, dtype=FP16)
+    pool = upload_pool(pp)
+    tok = _zipf(rng, T, N, 1.0)
+    x = torch.randn(T, H, device="cuda", dtype=torch.float16)
+    y0 = torch.randn(T, H, device="cuda", dtype=torch.float16)
+    t = torch.from_numpy(tok).cuda()
+
+    def run(xx, tt, yy0, group):
+        y = yy0.clone()
+        plan = plan_decode(tt, pool, group=group) if group else None
+        bgmv([y], [xx], pool, 0, ["p"], tt, plan=plan)
+        return y
+
+    say("bgmv full-size: direct vs grouped")
+    y_direct = run(x, t, y0, 0)
+    y_g4 = run(x, t, y0, 4)
+    y_g8 = run(x, t, y0, 8)
+    torch.cuda.synchronize()
+    for other in (y_g4, y_g8):
+        assert torch.allclose(other.float(), y_direct.float(), rtol=RTOL, atol=ATOL)
+    # a token's result does not depend on which other tokens share its work item: same summation order
+    assert torch.equal(y_g4, y_direct) and torch.equal(y_g8, y_direct)
+    say("bgmv full-size: token permutation")
+    perm = torch.randperm(T, device="cuda")
+    y_perm = run(x[perm].contiguous(), t[perm].contiguous(), y0[perm].contiguous(), 4)
+    assert torch.equal(y_perm, y_g4[perm])
+    say("bgmv full-size: lora_apply")
+    y_api = lora_apply(y0.clone(), x, t, pool, 0, "p")
+    torch.cuda.synchronize()
+    assert torch.equal(y_api, y_direct)
+    say("bgmv full-size: page placement")
+    pp2 = PagedPool(np.random.default_rng(7), [16] * N, H, H, page_rows=8, dtype=FP16, extra_pages=9)
+    for i in range(N):
+        pp2.a_rows[pp2.rows(i)] = pp.a_rows[pp.rows(i)]
+        pp2.b_rows[pp2.rows(i)] = pp.b_rows[pp.rows(i)]
+    pool2 = upload_pool(pp2)
+    y2 = y0.clone()
+    bgmv([y2], [x], pool2, 0, ["p"], t, plan=plan_decode(t, pool2, group=4))
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y_g4)
+    say("bgmv full-size: linearity of the delta")
+    d1 = torch.zeros_like(y0)
+    d2 = torch.zeros_like(y0)
+    bgmv([d1], [x], pool, 0, ["p"], t, accumulate=False)
+    bgmv([d2], [(2 * x).contiguous()], pool, 0, ["p"], t, accumulate=False)
+    torch.cuda.synchronize()
+    normal = d1.abs() >= 2.0 ** -13
+    assert torch.equal(d2[normal], 2 * d1[normal])

@@ -1,0 +1,122 @@
+"""Pins the oracle's integer work (gather, grouping, work lists, chunk plan) against numpy closed
+forms and brute force.  None of these re-type the oracle's loops: they use argsort / unique /
+explicit enumeration."""
+import numpy as np
+import pytest
+from hypothesis import given, settings, strategies as st
+
+from oracle import oracle as orc
+
+
+def _np_gather(tok, page_tbl, rank, scaling, page_rows):
+    T = len(tok)
+    N, mp = page_tbl.shape
+    valid = tok >= 0
+    a = np.where(valid, tok, 0)
+    r = np.where(valid, rank[a], 0)
+    npg = -(-r // page_rows)
+    p = np.arange(mp)[None, :]
+    off = np.where(valid[:, None] & (p < npg[:, None]), page_tbl[a] * page_rows, -1)
+    return off.astype(np.int32), r.astype(np.int32), np.where(valid, scaling[a], 0).astype(np.float32)
+
+
+@pytest.mark.parametrize("page_rows", [1, 8, 16])
+def test_pool_gather_closed_form(page_rows):
+    rng = np.random.default_rng(page_rows)
+    N, T = 37, 300
+    rank = rng.choice([1, 3, 8, 16, 24, 32, 64], N).astype(np.int32)
+    mp = -(-64 // page_rows)
+    page_tbl = rng.integers(0, 5000, (N, mp)).astype(np.int32)
+    scaling = rng.random(N).astype(np.float32)
+    tok = rng.integers(-1, N, T).astype(np.int32)
+    got = orc.pool_gather(tok, page_tbl, rank, scaling, page_rows)
+    want = _np_gather(tok, page_tbl, rank, scaling, page_rows)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+
+
+def test_pool_gather_rejects_out_of_range():
+    page_tbl = np.zeros((4, 2), np.int32)
+    with pytest.raises(IndexError):
+        orc.pool_gather(np.array([0, 4], np.int32), page_tbl, np.ones(4, np.int32), np.ones(4, np.float32), 8)
+    with pytest.raises(IndexError):   # rank needs more pages than the table has
+        orc.pool_gather(np.array([0], np.int32), page_tbl, np.full(4, 17, np.int32), np.ones(4, np.float32), 8)
+
+
+def _np_segments(tok, n_adapters):
+    key = np.where(tok >= 0, tok, n_adapters)
+    perm = np.argsort(key, kind="stable").astype(np.int32)
+    valid = tok[tok >= 0]
+    ad, cnt = np.unique(valid, return_counts=True)
+    start = np.concatenate([[0], np.cumsum(cnt)[:-1]]) if len(cnt) else np.zeros(0)
+    return perm, start.astype(np.int32), cnt.astype(np.int32), ad.astype(np.int32), len(valid)
+
+
+@settings(max_examples=200, deadline=None)
+@given(st.lists(st.integers(-1, 11), min_size=0, max_size=80))
+def test_build_segments_vs_argsort(toks):
+    tok = np.array(toks, np.int32)
+    perm, ss, sl, sa, nv = orc.build_segments(tok, 12)
+    wperm, wss, wsl, wsa, wnv = _np_segments(tok, 12)
+    assert np.array_equal(perm, wperm) and np.array_equal(ss, wss) and np.array_equal(sl, wsl)
+    assert np.array_equal(sa, wsa) and nv == wnv
+
+
+def test_build_segments_empty_and_single():
+    perm, ss, sl, sa, nv = orc.build_segments(np.zeros(0, np.int32), 4)
+    assert perm.size == 0 and ss.size == 0 and nv == 0
+    perm, ss, sl, sa, nv = orc.build_segments(np.array([3], np.int32), 4)
+    assert perm.tolist() == [0] and ss.tolist() == [0] and sl.tolist() == [1] and sa.tolist() == [3] and nv == 1
+    with pytest.raises(IndexError):
+        orc.build_segments(np.array([4], np.int32), 4)
+
+
+@settings(max_examples=150, deadline=None)
+@given(st.lists(st.integers(-1, 6), min_size=0, max_size=60), st.sampled_from([1, 2, 4, 8]))
+def test_build_chunks_brute_force(toks, group):
+    tok = np.array(toks, np.int32)
+    T = len(tok)
+    perm, ss, sl, sa, nv = orc.build_segments(tok, 7)
+    cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, T, group)
+    # brute force over sorted positions: a new chunk starts when the adapter changes or the
+    # running chunk already holds `group` tokens
+    key = [int(tok[p]) if tok[p] >= 0 else -1 for p in perm]
+    want = []
+    for i, k in enumerate(key):
+        if want and want[-1][2] == k and want[-1][1] < group:
+            want[-1][1] += 1
+        else:
+            want.append([i, 1, k])
+    assert [list(map(int, c)) for c in zip(cs, cl, ca)] == want
+    assert int(cl.sum()) == T
+    assert len(cs) <= max(T, 1)
+
+
+def test_sgmv_plan_brute_force():
+    rng = np.random.default_rng(5)
+    lens = rng.integers(0, 400, 23)
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    ts, t0, tn = orc.sgmv_plan(starts, lens, 64)
+    want = [(s, int(starts[s]) + o, min(64, int(lens[s]) - o)) for s in range(23) for o in range(0, int(lens[s]), 64)]
+    assert list(zip(ts.tolist(), t0.tolist(), tn.tolist())) == want
+    covered = np.zeros(int(lens.sum()), int)
+    for _, a, n in want:
+        covered[a:a + n] += 1
+    assert np.all(covered == 1)
+
+
+@pytest.mark.parametrize("batch,tkn,cap", [(1, 64, 8), (3, 20, 8), (2, 8, 8), (4, 1, 16), (2, 17, 16), (1, 256, 8)])
+def test_cpu_chunk_plan_matches_reference_formulas(batch, tkn, cap):
+    req, tok0, ntok = orc.cpu_chunk_plan(batch, tkn, cap)
+    # lightllm/models/lora_cpu.py:150-151,210-213: cpu_per_request and the last chunk's size
+    cpr = (tkn - 1) // cap + 1
+    last = tkn % cap if tkn % cap > 0 else cap
+    assert len(req) == batch * cpr
+    for row_id in range(batch * cpr):
+        b, off = divmod(row_id, cpr)             # app.py:133-134 dim_0, dim_1
+        assert req[row_id] == b and tok0[row_id] == off * cap
+        assert ntok[row_id] == (last if off == cpr - 1 else cap)
+    cover = np.zeros((batch, tkn), int)
+    for b, a, n in zip(req, tok0, ntok):
+        cover[b, a:a + n] += 1
+    assert np.all(cover == 1)
