@@ -332,13 +332,19 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
                 acc[nb] = mfma16<DT>(vlo[ks], bop, acc[nb]);
             }
         }
-        // ---- wave-private transpose through LDS, then 16-byte row-contiguous y update
+        // ---- transpose through LDS (one 16 x TN tile per wavefront), then 16-byte row-contiguous y update
+        {
+            // volatile: one ds_write_b32 per element.  Left to itself the compiler pairs these
+            // stores into ds_write2_b32 and, in the variant without the B staging tile, gets two
+            // of the paired offsets wrong.
+            typedef __attribute__((address_space(3))) volatile float lds_vfloat;
+            lds_vfloat *so = (lds_vfloat *)&s_out[wave][4 * g][m];
 #pragma unroll
-        for (int nb = 0; nb < NBC; nb++)
+            for (int nb = 0; nb < NBC; nb++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) s_out[wave][4 * g + i][nb * 16 + m] = acc[nb][i];
-        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): LDS writes of this wavefront are done
-        __builtin_amdgcn_wave_barrier();
+                for (int i = 0; i < 4; i++) so[i * OPITCH + nb * 16] = acc[nb][i];
+        }
+        __syncthreads();
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int pp = lane + 64 * q, t = pp >> 4, c = pp & 15;
@@ -359,8 +365,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
                 stg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col, pack8<DT>(o));
             }
         }
-        __builtin_amdgcn_s_waitcnt(0xc07f);
-        __builtin_amdgcn_wave_barrier();
+        if constexpr (BT) __syncthreads();   // staging tile is rewritten by the next step (the B staging barrier covers !BT)
     }
 }
 

@@ -203,7 +203,7 @@ def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: 
 
 
 def lora_prefill_ref(x: torch.Tensor, A_T: torch.Tensor, B_T: torch.Tensor, layer_idx: int,
-                     workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The reference's prefill expression on its own layout (``lora_gpu.py:125-128``):
     ``torch.bmm(torch.bmm(x, A_T[:bsz, layer].transpose(-1,-2)), B_T[:bsz, layer].transpose(-1,-2))``
     with x [bsz, Lpad, Hin], A_T [>=bsz, L, r, Hin], B_T [>=bsz, L, Hout, r]; request b uses slot b."""
@@ -216,7 +216,12 @@ def lora_prefill_ref(x: torch.Tensor, A_T: torch.Tensor, B_T: torch.Tensor, laye
         raise ValueError("x, A_T and B_T shapes do not fit the reference prefill call")
     if not (x.dtype == A_T.dtype == B_T.dtype):
         raise TypeError("x and the pool must share one 16-bit dtype")
-    y = torch.empty((bsz, lpad, hout), dtype=x.dtype, device=x.device)
+    if out is None:
+        y = torch.empty((bsz, lpad, hout), dtype=x.dtype, device=x.device)
+    else:
+        y = out
+        if tuple(y.shape) != (bsz, lpad, hout) or y.dtype != x.dtype or not y.is_contiguous() or not y.is_cuda:
+            raise ValueError("out must be a contiguous device tensor [bsz, Lpad, Hout] of x's dtype")
     if workspace is None:
         workspace = sgmv_workspace(bsz * lpad, bsz, x.device)
     rc = _ext.lib().mlora_prefill_reflayout(y.data_ptr(), x.data_ptr(), A_T.data_ptr(), B_T.data_ptr(), bsz, lpad, L, r,

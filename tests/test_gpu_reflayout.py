@@ -1,0 +1,94 @@
+"""GPU parity on the reference's own pool layout and call signatures (lightllm/models/lora_gpu.py)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import ATOL, RTOL, assert_close_bits, say
+from helpers import BF16, FP16, bits_of, bits_to_torch, f32_of, torch_to_bits
+from mlora import Lora_GPU, add_lora_bgmv, lora_prefill_ref
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("N,L,r,hin,hout,T,layer,scale,dtype", [
+    (24, 4, 64, 4096, 4096, 17, 2, 1.0, FP16),       # the shipped shapes (rank 64, hidden 4096), fewer layers
+    (8, 2, 16, 4096, 4096, 32, 0, 2.0, FP16),        # config 1
+    (5, 3, 16, 512, 1536, 9, 1, 0.5, BF16),
+    (4, 2, 12, 256, 264, 6, 1, 1.0, FP16),           # rank not a multiple of 8
+    (3, 1, 2, 128, 128, 5, 0, 1.0, FP16),            # the CPU worker's default rank
+])
+def test_add_lora_bgmv_vs_oracle(N, L, r, hin, hout, T, layer, scale, dtype):
+    rng = np.random.default_rng(N * 100 + r)
+    wa = bits_of((rng.standard_normal((N, L, r, hin)) * 0.02).astype(np.float32), dtype)
+    wb = bits_of((rng.standard_normal((N, L, hout, r)) * 0.02).astype(np.float32), dtype)
+    idx = rng.integers(0, N, T).astype(np.int64)
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype)
+    y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), dtype)
+    want = y0.copy()
+    orc.add_lora_bgmv_ref(want, x, wa, wb, idx, layer, scale, dtype)
+    y = bits_to_torch(y0, dtype, "cuda")
+    say(f"add_lora_bgmv N={N} L={L} r={r} {hin}x{hout} T={T}")
+    add_lora_bgmv(y, bits_to_torch(x, dtype, "cuda"), bits_to_torch(wa, dtype, "cuda"), bits_to_torch(wb, dtype, "cuda"),
+                  torch.from_numpy(idx).cuda(), layer, scale)
+    torch.cuda.synchronize()
+    assert_close_bits(torch_to_bits(y), want, dtype)
+
+
+def test_add_lora_bgmv_bad_index_leaves_row_untouched():
+    rng = np.random.default_rng(3)
+    N, L, r, H, T = 4, 1, 8, 128, 6
+    wa = torch.randn(N, L, r, H, device="cuda", dtype=torch.float16)
+    wb = torch.randn(N, L, H, r, device="cuda", dtype=torch.float16)
+    x = torch.randn(T, H, device="cuda", dtype=torch.float16)
+    y0 = torch.randn(T, H, device="cuda", dtype=torch.float16)
+    idx = torch.tensor([0, 4, 1, -1, 31, 3], device="cuda")     # 4, -1, 31 are outside the pool
+    y = y0.clone()
+    say("add_lora_bgmv with out-of-range indices")
+    add_lora_bgmv(y, x, wa, wb, idx, 0, 1.0)
+    torch.cuda.synchronize()
+    bad = torch.tensor([False, True, False, True, True, False], device="cuda")
+    assert torch.equal(y[bad], y0[bad])
+    assert not torch.equal(y[~bad], y0[~bad])
+
+
+@pytest.mark.parametrize("B,Lpad,L,r,hin,hout,layer,dtype", [
+    (3, 64, 2, 64, 4096, 4096, 1, FP16),
+    (4, 37, 3, 16, 512, 768, 2, BF16),
+    (1, 130, 1, 8, 256, 256, 0, FP16),
+])
+def test_prefill_ref_vs_oracle(B, Lpad, L, r, hin, hout, layer, dtype):
+    rng = np.random.default_rng(B * 10 + r)
+    A_T = bits_of((rng.standard_normal((B + 1, L, r, hin)) * 0.02).astype(np.float32), dtype)
+    B_T = bits_of((rng.standard_normal((B + 1, L, hout, r)) * 0.02).astype(np.float32), dtype)
+    x = bits_of(rng.standard_normal((B, Lpad, hin)).astype(np.float32), dtype)
+    want = orc.prefill_bmm_ref(x, A_T[:B], B_T[:B], layer, dtype, round_mid=False)
+    say(f"prefill ref B={B} Lpad={Lpad} r={r} {hin}x{hout}")
+    y = lora_prefill_ref(bits_to_torch(x, dtype, "cuda"), bits_to_torch(A_T, dtype, "cuda"),
+                         bits_to_torch(B_T, dtype, "cuda"), layer)
+    torch.cuda.synchronize()
+    assert_close_bits(torch_to_bits(y), want, dtype)
+
+
+def test_lora_gpu_mirror_calls():
+    """The calls LlamaTransformerLayerInfer._get_qkv makes (transformer_layer_infer.py:76-81,101-111)."""
+    cfg = dict(n_layers=2, batch_size=12, lora_rank=16, hidden_dim=1024, tp_degree=1, max_prefill_batch_size=3,
+               mode=["aaas-cached"])
+    say("Lora_GPU mirror: decode and prefill through invoke_one_layer_{q,k,v}")
+    g = Lora_GPU(cfg)
+    assert g.q_down.shape == (12, 2, 16, 1024) and g.q_up.shape == (12, 2, 1024, 16)
+    x = torch.randn(5, 1024, device="cuda", dtype=torch.float16)
+    for name in "qkv":
+        y = getattr(g, f"invoke_one_layer_{name}")(x, 1, False)
+        inds = g.select_inds[4]
+        down, up = getattr(g, f"{name}_down"), getattr(g, f"{name}_up")
+        want = torch.stack([x[i].float() @ down[inds[i], 1].float().t() @ up[inds[i], 1].float().t() for i in range(5)])
+        assert y.shape == (5, 1024) and torch.allclose(y.float(), want, rtol=RTOL, atol=ATOL)
+    xp = torch.randn(3, 20, 1024, device="cuda", dtype=torch.float16)
+    for name in "qkv":
+        y = getattr(g, f"invoke_one_layer_{name}")(xp, 0, True)
+        down, up = getattr(g, f"{name}_down_prefill"), getattr(g, f"{name}_up_prefill")
+        want = torch.bmm(torch.bmm(xp.float(), down[:3, 0].float().transpose(-1, -2)), up[:3, 0].float().transpose(-1, -2))
+        assert y.shape == (3, 20, 1024) and torch.allclose(y.float(), want, rtol=RTOL, atol=ATOL)
+    g.merge_lora_prefill(2, re_inds=[7, 3])
+    assert torch.equal(g.k_up[7], g.k_up_prefill[0]) and torch.equal(g.v_down[3], g.v_down_prefill[1])

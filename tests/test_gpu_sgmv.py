@@ -1,0 +1,140 @@
+"""GPU parity: SGMV prefill kernels (MFMA) through the C ABI against the fp32-accumulated oracle, and
+against the decode kernel at full config-4 size."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import ATOL, RTOL, assert_close_bits, oracle_apply, say, tdtype, upload_pool
+from helpers import BF16, FP16, PagedPool, bits_of, bits_to_torch, f32_of, torch_to_bits
+from mlora import bgmv, sgmv
+
+pytestmark = pytest.mark.gpu
+
+
+def _segments(lens, adapters):
+    lens = np.asarray(lens, np.int32)
+    start = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    return start, lens, np.asarray(adapters, np.int32)
+
+
+def _tok_of(start, lens, adapters, T):
+    tok = np.full(T, -1, np.int32)
+    for s, l, a in zip(start, lens, adapters):
+        tok[s:s + l] = a
+    return tok
+
+
+def _run(pp, x_bits, seg, y0_bits, accumulate=True):
+    pool = upload_pool(pp)
+    T = x_bits.shape[0]
+    x = bits_to_torch(x_bits, pp.dtype, "cuda")
+    y = bits_to_torch(y0_bits, pp.dtype, "cuda") if y0_bits is not None else \
+        torch.full((T, pp.hout), float("nan"), dtype=tdtype(pp.dtype), device="cuda")
+    ss, sl, sa = (torch.from_numpy(a).cuda() for a in seg)
+    sgmv(y, x, pool, 0, "p", ss, sl, sa, accumulate=accumulate)
+    torch.cuda.synchronize()
+    return torch_to_bits(y)
+
+
+CASES = [
+    # name, segment lengths, ranks of the pool, hin, hout, dtype
+    ("C4 slice q 5120x5120 bf16 r64", [70, 128, 1, 300, 64, 65], [64] * 8, 5120, 5120, BF16),
+    ("C4 slice gate 5120x13824 bf16 r64", [130, 33], [64] * 4, 5120, 13824, BF16),
+    ("C4 slice down 13824x5120 bf16 r64", [90, 17, 64], [64] * 4, 13824, 5120, BF16),
+    ("fp16 hetero ranks 4096x4096", [40, 100, 7, 64, 129], [8, 16, 32, 64, 24], 4096, 4096, FP16),
+    ("rank 16 pool 1024x2048", [63, 64, 65, 1], [16, 8, 16, 3], 1024, 2048, FP16),
+    ("odd widths 200x72 bf16", [5, 70], [32, 5], 200, 72, BF16),
+]
+
+
+@pytest.mark.parametrize("name,lens,ranks,hin,hout,dtype", CASES, ids=[c[0] for c in CASES])
+def test_sgmv_vs_oracle(name, lens, ranks, hin, hout, dtype):
+    import zlib
+    rng = np.random.default_rng(zlib.crc32(name.encode()))
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=dtype)
+    adapters = rng.integers(0, len(ranks), len(lens))
+    seg = _segments(lens, adapters)
+    T = int(np.sum(lens))
+    tok = _tok_of(*seg, T)
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype)
+    y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), dtype)
+    say(f"sgmv {name} accumulate")
+    got = _run(pp, x, seg, y0)
+    assert_close_bits(got, oracle_apply(pp, x, tok, y0), dtype, name)
+    say(f"sgmv {name} delta")
+    got_d = _run(pp, x, seg, None, accumulate=False)
+    want_d = oracle_apply(pp, x, tok, None)
+    assert_close_bits(got_d, want_d, dtype, name + " delta")
+    # the hi+lo split keeps the intermediate at fp32 accuracy: the delta is much closer to the
+    # fp64-accumulated oracle than a 16-bit intermediate would allow
+    want64 = f32_of(oracle_apply(pp, x, tok, None, acc64=True), dtype).astype(np.float64)
+    err = np.abs(f32_of(got_d, dtype) - want64)
+    mant = 10 if dtype == FP16 else 7
+    assert np.all(err <= 2.0 ** -mant * np.abs(want64) + 1e-5), "delta is not within one ulp of the exact result"
+
+
+def test_sgmv_integer_inputs_bit_exact():
+    rng = np.random.default_rng(71)
+    ranks = [8, 16, 3, 64, 5]
+    pp = PagedPool(rng, ranks, hin=512, hout=384, page_rows=8, dtype=FP16, integer=True)
+    pp.scaling[:] = [1, 2, 0.5, -1, 4]
+    lens = [64, 3, 100, 65, 1]
+    seg = _segments(lens, [3, 0, 1, 2, 4])
+    T = sum(lens)
+    tok = _tok_of(*seg, T)
+    xi = (rng.integers(-2, 3, (T, 512)) * (rng.random((T, 512)) < 0.05)).astype(np.float32)
+    y0 = bits_of(rng.integers(-8, 9, (T, 384)).astype(np.float32), FP16)
+    x = bits_of(xi, FP16)
+    want = oracle_apply(pp, x, tok, y0)
+    assert np.abs(f32_of(want, FP16)).max() < 2048
+    say("sgmv integer-valued inputs")
+    assert np.array_equal(_run(pp, x, seg, y0), want)
+
+
+def test_sgmv_segments_without_adapter_and_gaps():
+    rng = np.random.default_rng(72)
+    pp = PagedPool(rng, [16, 32], 256, 256, page_rows=8, dtype=FP16)
+    # tokens 0..9 uncovered, then a segment with no adapter, an empty one, and two real ones
+    ss = np.array([10, 40, 40, 104], np.int32)
+    sl = np.array([30, 0, 64, 20], np.int32)
+    sa = np.array([-1, 1, 0, 1], np.int32)
+    T = 130
+    tok = _tok_of(ss, sl, sa, T)
+    x = bits_of(rng.standard_normal((T, 256)).astype(np.float32), FP16)
+    y0 = bits_of(rng.standard_normal((T, 256)).astype(np.float32), FP16)
+    say("sgmv gaps / adapter-less segment, accumulate")
+    got = _run(pp, x, (ss, sl, sa), y0)
+    assert np.array_equal(got[tok < 0], y0[tok < 0])
+    assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16)
+    say("sgmv gaps / adapter-less segment, delta")
+    got_d = _run(pp, x, (ss, sl, sa), None, accumulate=False)
+    assert np.all(got_d[10:40] == 0)                       # adapter-less segment is defined as zeros
+    covered = tok >= 0
+    assert_close_bits(got_d[covered], oracle_apply(pp, x, tok, None)[covered], FP16)
+
+
+def test_sgmv_equals_bgmv_at_config4_size():
+    """Config 4 at full size (16 requests, lengths U[128,1024], 32 rank-64 adapters, hidden 5120, bf16):
+    the prefill kernels and the decode kernel must agree within tolerance on every token."""
+    rng = np.random.default_rng(1004)
+    lens = rng.integers(128, 1025, 16)
+    adapters = rng.integers(0, 32, 16)
+    seg = _segments(lens, adapters)
+    T = int(lens.sum())
+    pp = PagedPool(rng, [64] * 32, 5120, 5120, page_rows=8, dtype=BF16)
+    pool = upload_pool(pp)
+    x = (torch.randn(T, 5120, device="cuda")).to(torch.bfloat16)
+    y0 = (torch.randn(T, 5120, device="cuda")).to(torch.bfloat16)
+    tok = torch.from_numpy(_tok_of(*seg, T)).cuda()
+    ys, yb = y0.clone(), y0.clone()
+    say(f"sgmv vs bgmv at config-4 size T={T}")
+    sgmv(ys, x, pool, 0, "p", *(torch.from_numpy(a).cuda() for a in seg))
+    bgmv([yb], [x], pool, 0, ["p"], tok)
+    torch.cuda.synchronize()
+    assert torch.allclose(ys.float(), yb.float(), rtol=RTOL, atol=ATOL)
+    # linearity of the delta in x at full size
+    d1, d2 = torch.zeros_like(y0), torch.zeros_like(y0)
+    sgmv(d1, x, pool, 0, "p", *(torch.from_numpy(a).cuda() for a in seg), accumulate=False)
+    sgmv(d2, (2 * x).contiguous(), pool, 0, "p", *(torch.from_numpy(a).cuda() for a in seg), accumulate=False)
+    torch.cuda.synchronize()
+    assert torch.equal(d2, 2 * d1)
