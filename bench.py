@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-LoRA decode hot path on one MI355X.
+
+Workload (the configuration the metric is quoted on): decode BGMV over the Llama-7B attention
+projections q/k/v/o (4096 -> 4096 each), 256 decode tokens, 64 rank-16 fp16 adapters in one paged
+pool, adapter per token ~ Zipf(1.0), scaling 2.0.  One step = one decode step's LoRA work: the
+adapter-pool gather once, then for each of the 32 layers one fused BGMV launch covering that
+layer's q, k, v (shared input) and o (own input), accumulating into the base projection outputs.
+Every layer has its own pool slabs, inputs and outputs (about 2.4 GB in all), so a step streams
+from HBM rather than from the 256 MB last-level cache.
+
+Prints one JSON line: throughput in token-projections/s, the HBM roofline of the BGMV kernel
+(algorithmic bytes / measured launch duration) and the CPU baseline (the CPU-assisted path's
+arithmetic timed on the host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "ae-296_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(T, projs, ranks_of_unique, elt=2):
+    """Per projection call: x read + y read and write + every touched adapter's rows once + indices."""
+    total = 0
+    for hin, hout in projs:
+        total += T * hin * elt + 2 * T * hout * elt + int(sum(ranks_of_unique)) * (hin + hout) * elt + 4 * T
+    return total
+
+
+def cpu_baseline(seconds=12.0):
+    """The reference's CPU-assisted LoRA arithmetic (x.float() @ down @ up -> half, one task per
+    request chunk) on config 1: 32 tokens, 8 rank-16 adapters, 4096 -> 4096, timed on the host cores."""
+    import numpy as np
+    from oracle import oracle as orc
+    rng = np.random.default_rng(1001)
+    T, N, r, H = 32, 8, 16, 4096
+    down = (rng.standard_normal((N, H, r)) * 0.02).astype(np.float32)
+    up = (rng.standard_normal((N, r, H)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((T, H)).astype(np.float16).view(np.uint16)
+    req_adapter = rng.integers(0, N, T).astype(np.int32)
+    cores = max(1, min(16, os.cpu_count() or 1))
+    orc.cpu_lora_batch(x, down, up, req_adapter, 1, 8, cores)          # warm-up
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        orc.cpu_lora_batch(x, down, up, req_adapter, 1, 8, cores)
+        n += 1
+    dt = time.perf_counter() - t0
+    return {"value": T * n / dt, "unit": "token-projections/s", "cores": cores, "kind": "port",
+            "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights), {n} repetitions "
+                      f"in {dt:.1f} s, one task per token over {cores} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import mlora
+    from mlora import workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    mlora._ext.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = args.layers
+    log(f"building config 2 with {L} layers ...")
+    wl = workloads.config2(n_layers=L, device=dev)
+    pool, T = wl.pool, len(wl.tok_adapter)
+    projs = ["q", "k", "v", "o"]
+    tok = torch.from_numpy(wl.tok_adapter).to(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2002)
+    x_qkv = [torch.randn(T, 4096, device=dev, generator=gen).half() for _ in range(L)]
+    x_o = [torch.randn(T, 4096, device=dev, generator=gen).half() for _ in range(L)]
+    ys = [[torch.randn(T, 4096, device=dev, generator=gen).half() for _ in projs] for _ in range(L)]
+    plan = mlora.plan_decode(tok, pool, group=args.group) if args.group else None
+
+    def bgmv_layers():
+        for l in range(L):
+            mlora.bgmv(ys[l], [x_qkv[l], x_qkv[l], x_qkv[l], x_o[l]], pool, l, projs, tok, plan=plan)
+
+    def step():
+        if plan is not None:
+            mlora.plan_decode(tok, pool, group=args.group, out=plan)
+        bgmv_layers()
+
+    step()
+    torch.cuda.synchronize()
+
+    def make_runner(fn):
+        if args.no_graph:
+            return fn
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            fn()
+        return g.replay
+
+    def timed(run, reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1)          # ms, on the stream the kernels run on
+
+    run_step = make_runner(step)
+    for _ in range(args.warmup):
+        run_step()
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter()
+    ms = timed(run_step, args.steps)
+    wall = time.perf_counter() - t_wall
+    ms_per_step = ms / args.steps
+    value = T * len(projs) * L / (ms_per_step * 1e-3)
+
+    # The dominant kernel alone: the same 32 launches without the gather, for the roofline figure.
+    run_bgmv = make_runner(bgmv_layers)
+    for _ in range(args.warmup):
+        run_bgmv()
+    ms_k = timed(run_bgmv, args.steps)
+    launch_us = ms_k * 1e3 / (args.steps * L)
+    uniq = np.unique(wl.tok_adapter[wl.tok_adapter >= 0])
+    alg = algorithmic_bytes(T, [pool.projections[p] for p in projs], wl.ranks[uniq])
+    achieved = alg / (launch_us * 1e-6) / 1e9
+    per_token_gather = sum(T * h[0] * 2 + 2 * T * h[1] * 2 + int(wl.ranks[wl.tok_adapter].sum()) * (h[0] + h[1]) * 2 + 4 * T
+                           for h in (pool.projections[p] for p in projs))
+
+    out = {
+        "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",
+        "value": value, "unit": "token-projections/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "config 2: decode BGMV, Llama-7B q/k/v/o 4096->4096, 256 tokens, 64 rank-16 adapters, "
+                               "Zipf(1.0), fp16, scaling 2.0",
+                   "layers": L, "projections_per_launch": len(projs), "launches_per_step": L + (1 if plan else 0),
+                   "tokens": T, "adapters": 64, "adapters_touched": int(len(uniq)), "group": args.group,
+                   "hip_graph": not args.no_graph, "wall_s_timed_region": wall},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "bgmv_kernel (4 projections per launch)", "launch_us": launch_us,
+                     "algorithmic_bytes_per_launch": alg, "per_token_gather_bytes_per_launch": per_token_gather},
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu:
+        log("timing the CPU baseline ...")
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
