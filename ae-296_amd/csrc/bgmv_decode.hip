@@ -30,7 +30,7 @@ __device__ __forceinline__ int pool_row(const int32_t *__restrict__ tbl, long lo
     return (row < 0 || row >= n_rows) ? -1 : (int)row;
 }
 
-template <int DT, int G, int RMAX, int NT, bool BT>
+template <int DT, int G, int RMAX, int NT, bool BT, bool PF>
 __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 {
     constexpr int NW = NT / 64;
@@ -119,6 +119,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
     __syncthreads();
 
+    if (p.dbg_stop == 1) return;
     // ---------------------------------------------------------------- shrink
     // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot
     // beyond ntok reads token 0 (both discarded below), a column chunk past the end of the
@@ -144,8 +145,13 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll
         for (int i = 0; i < RPG; i++) acc[k][i] = 0.f;
 
-#pragma unroll 1
-    for (int it0 = 0; it0 < n_it; it0 += U) {
+    // Prefetch for the expand (PF): the B rank rows (first EB of them) and the y rows of this lane's
+    // first output chunk are requested right behind the first round of A/x loads, so their latency
+    // is hidden behind the shrink instead of starting after the reduction.
+    uint4 bpre[PF ? EB : 1];
+    uint4 ypre[PF ? G : 1];
+    const bool pf_active = PF && !BT && tid < ncc_out;
+    auto shrink_round = [&](int it0, bool first) {
         uint4 xv[G][U];
         uint4 av[RPG][U];
         bool cv[U];
@@ -159,6 +165,18 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll
             for (int i = 0; i < RPG; i++) av[i][u] = ap[i][cs];
         }
+        if constexpr (PF && !BT) {
+            if (first && pf_active) {
+#pragma unroll
+                for (int jj = 0; jj < EB; jj++) {
+                    const int row = __builtin_amdgcn_readfirstlane(s_brow[jj]);
+                    bpre[jj] = row >= 0 ? ldg16(brows + (size_t)row * hout + (size_t)tid * 8) : zero16();
+                }
+#pragma unroll
+                for (int k = 0; k < G; k++)
+                    ypre[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)tid * 8) : zero16();
+            }
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -166,11 +184,24 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
                 xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
                 xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
             }
+            if (p.dbg_stop == 3) {      // experiments only: loads without the dot products
+#pragma unroll
+                for (int i = 0; i < RPG; i++)
+#pragma unroll
+                    for (int k = 0; k < G; k++)
+                        acc[k][i] += __builtin_bit_cast(float, (av[i][u].x ^ av[i][u].y ^ av[i][u].z ^ av[i][u].w ^ xv[k][u].x ^ xv[k][u].w) & 0x3fffffffu);
+                continue;
+            }
 #pragma unroll
             for (int i = 0; i < RPG; i++)
 #pragma unroll
                 for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
         }
+    };
+    if (p.dbg_stop != 4) {
+        shrink_round(0, true);
+#pragma unroll 1
+        for (int it0 = U; it0 < n_it; it0 += U) shrink_round(it0, false);
     }
 #pragma unroll
     for (int k = 0; k < G; k++)
@@ -193,15 +224,21 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
     __syncthreads();
 
+    if (p.dbg_stop == 3) { if (acc[0][0] == 12345.678f) y[0] = 1; return; }
+    if (p.dbg_stop == 2) { if (tid == 0 && s_v[0][0] == 12345.678f) y[0] = 1; return; }
     // ---------------------------------------------------------------- expand
     if constexpr (!BT) {
 #pragma unroll 1
         for (int cc = tid; cc < ncc_out; cc += NT) {
+            const bool pre = PF && cc == tid;            // this step's first rows and y are already in registers
             float o[G][8];
 #pragma unroll
             for (int k = 0; k < G; k++) {
-                if (p.accumulate && tok[k] >= 0) unpack8<DT>(ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8), o[k]);
-                else {
+                if (p.accumulate && tok[k] >= 0) {
+                    uint4 yv;
+                    if (PF && pre) yv = ypre[k]; else yv = ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8);
+                    unpack8<DT>(yv, o[k]);
+                } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) o[k][e] = 0.f;
                 }
@@ -209,10 +246,15 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll 1
             for (int j0 = 0; j0 < r; j0 += EB) {
                 uint4 bv[EB];
+                if (PF && pre && j0 == 0) {
 #pragma unroll
-                for (int jj = 0; jj < EB; jj++) {
-                    const int row = __builtin_amdgcn_readfirstlane(s_brow[j0 + jj]);
-                    bv[jj] = row >= 0 ? ldg16(brows + (size_t)row * hout + (size_t)cc * 8) : zero16();
+                    for (int jj = 0; jj < EB; jj++) bv[jj] = bpre[jj];
+                } else {
+#pragma unroll
+                    for (int jj = 0; jj < EB; jj++) {
+                        const int row = __builtin_amdgcn_readfirstlane(s_brow[j0 + jj]);
+                        bv[jj] = row >= 0 ? ldg16(brows + (size_t)row * hout + (size_t)cc * 8) : zero16();
+                    }
                 }
 #pragma unroll
                 for (int jj = 0; jj < EB; jj++) {
@@ -292,13 +334,13 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
 }
 
-template <int DT, int G, int RMAX, int NT, bool BT>
+template <int DT, int G, int RMAX, int NT, bool BT, bool PF = false>
 static int launch_one(const BgmvArgs &a, hipStream_t s)
 {
     const long long total = (long long)a.n_proj * a.items_per_proj;
     const unsigned grid = (unsigned)(((total + 7) / 8) * 8);
     if (grid == 0) return 0;
-    hipLaunchKernelGGL((bgmv_kernel<DT, G, RMAX, NT, BT>), dim3(grid), dim3(NT), 0, s, a);
+    hipLaunchKernelGGL((bgmv_kernel<DT, G, RMAX, NT, BT, PF>), dim3(grid), dim3(NT), 0, s, a);
     return (int)hipGetLastError();
 }
 

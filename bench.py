@@ -64,6 +64,64 @@ def cpu_baseline(seconds=12.0):
                       f"in {dt:.1f} s, one task per token over {cores} threads"}
 
 
+def bench_c4(args, dev):
+    """Prefill SGMV, config 4: Llama-13B shapes (hidden 5120, MLP 13824), 16 requests with prompt lengths
+    U[128, 1024], each bound to one of 32 rank-64 adapters, bf16, tokens packed per request.  One step =
+    the seven projections of one layer (q, k, v, o, gate, up, down), each one mlora_sgmv call."""
+    import numpy as np
+    import torch
+
+    import mlora
+    from mlora import workloads
+    rng = np.random.default_rng(1004)
+    lens = rng.integers(128, 1025, 16).astype(np.int32)
+    adapters = rng.integers(0, 32, 16).astype(np.int32)
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    T = int(lens.sum())
+    projections = workloads.LLAMA13B_ALL
+    pool = mlora.AdapterPool(1, projections, 32, 32 * 8, page_rows=8, max_rank=64, dtype=torch.bfloat16, device=dev)
+    workloads.fill_pool(pool, np.full(32, 64, np.int32), np.full(32, 0.5, np.float32), rng, seed=1004)
+    ss, sl, sa = (torch.from_numpy(a).to(dev) for a in (starts, lens, adapters))
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4004)
+    x = {h: torch.randn(T, h, device=dev, generator=gen).bfloat16() for h in (5120, 13824)}
+    y = {p: torch.randn(T, projections[p][1], device=dev, generator=gen).bfloat16() for p in projections}
+    ws = mlora.sgmv_workspace(T, 16, dev)
+
+    def step():
+        for p, (hin, hout) in projections.items():
+            mlora.sgmv(y[p], x[hin], pool, 0, p, ss, sl, sa, accumulate=True, workspace=ws)
+
+    step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    flops = sum(2.0 * 64 * (hin + hout) * T for hin, hout in projections.values())
+    uniq = np.unique(adapters)
+    alg = sum(T * hin * 2 + 2 * T * hout * 2 + len(uniq) * 64 * (hin + hout) * 2 + 4 * T + 12 * 16
+              for hin, hout in projections.values())
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    gbs = alg / (ms_per_step * 1e-3) / 1e9
+    out = {"metric": "SGMV prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
+                                  "32 rank-64 adapters, bf16", "tokens": T, "segments": 16},
+           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                        "traffic": None, "kernel": "sgmv plan+shrink+reduce+expand, 7 projections",
+                        "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
+           "cpu_baseline": None}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -73,6 +131,10 @@ def main():
     ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
+    ap.add_argument("--workload", default="c2", choices=["c2", "c4"],
+                    help="c2 = decode BGMV (the headline metric), c4 = prefill SGMV on Llama-13B shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -90,6 +152,15 @@ def main():
     mlora._ext.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.calib_copy:
+        src = torch.ones(128 << 20, dtype=torch.float16, device=dev)      # 256 MiB read + 256 MiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.workload == "c4":
+        return bench_c4(args, dev)
     L = args.layers
     log(f"building config 2 with {L} layers ...")
     wl = workloads.config2(n_layers=L, device=dev)
