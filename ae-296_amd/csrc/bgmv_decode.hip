@@ -119,7 +119,6 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
     __syncthreads();
 
-    if (p.dbg_stop == 1) return;
     // ---------------------------------------------------------------- shrink
     // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot
     // beyond ntok reads token 0 (both discarded below), a column chunk past the end of the
@@ -184,25 +183,15 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
                 xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
                 xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
             }
-            if (p.dbg_stop == 3) {      // experiments only: loads without the dot products
-#pragma unroll
-                for (int i = 0; i < RPG; i++)
-#pragma unroll
-                    for (int k = 0; k < G; k++)
-                        acc[k][i] += __builtin_bit_cast(float, (av[i][u].x ^ av[i][u].y ^ av[i][u].z ^ av[i][u].w ^ xv[k][u].x ^ xv[k][u].w) & 0x3fffffffu);
-                continue;
-            }
 #pragma unroll
             for (int i = 0; i < RPG; i++)
 #pragma unroll
                 for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
         }
     };
-    if (p.dbg_stop != 4) {
-        shrink_round(0, true);
+    shrink_round(0, true);
 #pragma unroll 1
-        for (int it0 = U; it0 < n_it; it0 += U) shrink_round(it0, false);
-    }
+    for (int it0 = U; it0 < n_it; it0 += U) shrink_round(it0, false);
 #pragma unroll
     for (int k = 0; k < G; k++)
 #pragma unroll
@@ -224,8 +213,6 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
     __syncthreads();
 
-    if (p.dbg_stop == 3) { if (acc[0][0] == 12345.678f) y[0] = 1; return; }
-    if (p.dbg_stop == 2) { if (tid == 0 && s_v[0][0] == 12345.678f) y[0] = 1; return; }
     // ---------------------------------------------------------------- expand
     if constexpr (!BT) {
 #pragma unroll 1

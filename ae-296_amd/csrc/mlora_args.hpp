@@ -45,7 +45,6 @@ struct BgmvArgs {
     int n_proj;
     int items_per_proj;            // work-item bound per projection (T)
     int accumulate;
-    int dbg_stop;                  // experiments only: 1 = stop after the prologue, 2 = after the shrink
 };
 
 struct GatherArgs {
