@@ -3,13 +3,23 @@
 // same adapter (G = 1: one token per workgroup), so an adapter's rows are fetched once
 // per item and the rank-r intermediate never leaves the CU (fp32 in LDS).
 //
+// Work items come in two forms:
+//   - work records written by the gather kernel (WORK = true): one 320-byte record per
+//     workgroup holding the tokens, the adapter's rank, scaling and the row index of every
+//     rank row, already placed in launch order -- one dependent load before the streaming
+//     starts, no table walk, no barrier;
+//   - the plain form (WORK = false): workgroup t serves token t and walks the page table
+//     (or the dense reference layout) itself.
+//
 // Shrink: a wavefront is split into four 16-lane DPP rows.  Each 16-lane row reads
 // 256 contiguous bytes (two 128-byte lines) of one rank row per load, rank rows are
 // dealt round-robin to the four lane rows, and wavefronts split the Hin columns.  The
 // per-lane partial dot products are reduced with four DPP adds inside the 16-lane row
 // and across wavefronts through LDS.
 // Expand: every lane owns 8 contiguous output columns, so a wavefront reads 1 KiB
-// contiguous from each B rank row and writes y with 16-byte stores.
+// contiguous from each B rank row and writes y with 16-byte stores.  The first B rows and
+// the y rows of a lane's first output chunk are requested before the reduction, into the
+// registers the A rows have just vacated, so the expand does not start on a cold pipe.
 //
 // Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
 #include "mlora_args.hpp"
@@ -30,7 +40,7 @@ __device__ __forceinline__ int pool_row(const int32_t *__restrict__ tbl, long lo
     return (row < 0 || row >= n_rows) ? -1 : (int)row;
 }
 
-template <int DT, int G, int RMAX, int NT, bool BT, bool PF>
+template <int DT, int G, int RMAX, int NT, bool BT, bool WORK, bool PF = !BT>
 __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 {
     constexpr int NW = NT / 64;
@@ -40,40 +50,40 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     constexpr int EB = RMAX < 16 ? RMAX : 16;                   // B rank rows in flight per lane
     __shared__ float s_part[NW][G][RMAX];
     __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
-    __shared__ int s_arow[RMAX];
-    __shared__ int s_brow[RMAX];
+    __shared__ int s_arow[WORK ? 1 : RMAX];
+    __shared__ int s_brow[WORK ? 1 : RMAX];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = lane & 15, rg = lane >> 4;
     const PoolView &pv = p.pool;
 
-    // ---- work item.  Workgroups are dealt to the 8 XCDs round-robin by blockIdx, so give
-    // each XCD a contiguous range of items: neighbouring items of one projection (chunks of
-    // the same hot adapter) then share that XCD's L2.
-    int n_items = p.T;
-    if (p.chunk_start) { n_items = p.counters[2]; n_items = n_items < p.items_per_proj ? n_items : p.items_per_proj; }
-    const int total = p.n_proj * n_items;
-    const int per_xcd = (total + 7) >> 3;
-    const int slot = blockIdx.x >> 3;
-    const int w = (blockIdx.x & 7) * per_xcd + slot;
-    if (slot >= per_xcd || w >= total) return;
-    const int proj = w / n_items;
-    const int item = w - proj * n_items;
-
-    int ntok = 1, adapter;
+    int proj, ntok = 1, adapter, r;
+    float scale;
     int tok[G];
-    if (p.chunk_start) {
-        const int p0 = p.chunk_start[item];
-        ntok = p.chunk_len[item];
+    const int32_t *__restrict__ rows = nullptr;                 // WORK: row index of rank row j at rows[j]
+
+    if constexpr (WORK) {
+        // Records are stored in launch order: record b belongs to workgroup b of every projection.
+        // The gather interleaves consecutive chunks over the 8 XCDs (workgroups are dealt to XCDs
+        // round-robin by id), so the chunks of one hot adapter share one XCD's L2.
+        const int b = blockIdx.x % p.work_cap;
+        proj = blockIdx.x / p.work_cap;
+        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+        ntok = rec[0];
+        if (ntok <= 0) return;
         ntok = ntok < G ? ntok : G;
-        adapter = p.chunk_adapter[item];
+        adapter = rec[1];
+        r = rec[2];
+        scale = __builtin_bit_cast(float, rec[3]);
 #pragma unroll
         for (int k = 0; k < G; k++) {
-            int t = -1;
-            if (k < ntok && p0 + k >= 0 && p0 + k < p.T) t = p.perm[p0 + k];
+            const int t = k < ntok ? rec[4 + k] : -1;
             tok[k] = (t >= 0 && t < p.T) ? t : -1;
         }
+        rows = rec + WORK_ROWS_AT;
     } else {
+        const int item = blockIdx.x % p.T;
+        proj = blockIdx.x / p.T;
         tok[0] = item;
 #pragma unroll
         for (int k = 1; k < G; k++) tok[k] = -1;
@@ -82,8 +92,19 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             const long long a64 = p.tok_adapter64[item];
             adapter = (a64 < 0 || a64 >= pv.n_adapters) ? -2 : (int)a64;
         }
+        if (adapter >= pv.n_adapters) adapter = -2;
+        r = 0;
+        scale = 0.f;
+        if (adapter >= 0) {
+            r = pv.rank ? pv.rank[adapter] : pv.uniform_rank;
+            scale = pv.scaling ? pv.scaling[adapter] : pv.uniform_scale;
+            if (pv.a_tbl || pv.b_tbl) {
+                const int cap = pv.max_pages << pv.page_shift;
+                r = r > cap ? cap : r;
+            }
+        }
     }
-    if (adapter >= pv.n_adapters) adapter = -2;
+    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
 
     const int hin = p.hin[proj], hout = p.hout[proj];
     const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x[proj]);
@@ -104,20 +125,40 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
         return;
     }
 
-    int r = pv.rank ? pv.rank[adapter] : pv.uniform_rank;
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    if (pv.a_tbl || pv.b_tbl) {
-        const int cap = pv.max_pages << pv.page_shift;
-        r = r > cap ? cap : r;
+    if constexpr (!WORK) {
+        // Row index of every rank row, looked up once per work item (-1 = absent / out of bounds).
+        for (int j = tid; j < RMAX; j += NT) {
+            s_arow[j] = j < r ? pool_row(pv.a_tbl, pv.a_dense_stride, adapter, j, pv, pv.n_rows_a) : -1;
+            if constexpr (!BT) s_brow[j] = j < r ? pool_row(pv.b_tbl, pv.b_dense_stride, adapter, j, pv, pv.n_rows_b) : -1;
+        }
+        __syncthreads();
     }
-    const float scale = pv.scaling ? pv.scaling[adapter] : pv.uniform_scale;
-
-    // Row index of every rank row, looked up once per work item (-1 = absent / out of bounds).
-    for (int j = tid; j < RMAX; j += NT) {
-        s_arow[j] = j < r ? pool_row(pv.a_tbl, pv.a_dense_stride, adapter, j, pv, pv.n_rows_a) : -1;
-        if constexpr (!BT) s_brow[j] = j < r ? pool_row(pv.b_tbl, pv.b_dense_stride, adapter, j, pv, pv.n_rows_b) : -1;
-    }
-    __syncthreads();
+    // Row lookups.  Records hold -1 for every absent rank row, so record reads need no rank guard
+    // and are issued as plain (batched) loads.
+    auto a_row = [&](int j) -> int {
+        if constexpr (WORK) { const int row = rows[j]; return (row >= 0 && row < pv.n_rows_a) ? row : -1; }
+        else return s_arow[j];
+    };
+    auto b_rows_of = [&](int j0, int (&out)[EB]) {     // rows of rank rows j0 .. j0+EB-1 (wavefront-uniform)
+        if constexpr (WORK) {
+            if constexpr (EB % 4 == 0) {
+                const int4 *q = reinterpret_cast<const int4 *>(rows + j0);
+#pragma unroll
+                for (int m = 0; m < EB / 4; m++) {
+                    const int4 v = q[m];
+                    out[4 * m] = v.x; out[4 * m + 1] = v.y; out[4 * m + 2] = v.z; out[4 * m + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < EB; jj++) out[jj] = rows[j0 + jj];
+            }
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++) out[jj] = (out[jj] >= 0 && out[jj] < pv.n_rows_b) ? out[jj] : -1;
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++) out[jj] = __builtin_amdgcn_readfirstlane(s_brow[j0 + jj]);
+        }
+    };
 
     // ---------------------------------------------------------------- shrink
     // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot
@@ -131,7 +172,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     unsigned row_ok = 0;
 #pragma unroll
     for (int i = 0; i < RPG; i++) {
-        const int row = s_arow[rg + 4 * i];
+        const int row = a_row(rg + 4 * i);
         row_ok |= (row >= 0 ? 1u : 0u) << i;
         ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
     }
@@ -144,13 +185,8 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll
         for (int i = 0; i < RPG; i++) acc[k][i] = 0.f;
 
-    // Prefetch for the expand (PF): the B rank rows (first EB of them) and the y rows of this lane's
-    // first output chunk are requested right behind the first round of A/x loads, so their latency
-    // is hidden behind the shrink instead of starting after the reduction.
-    uint4 bpre[PF ? EB : 1];
-    uint4 ypre[PF ? G : 1];
-    const bool pf_active = PF && !BT && tid < ncc_out;
-    auto shrink_round = [&](int it0, bool first) {
+#pragma unroll 1
+    for (int it0 = 0; it0 < n_it; it0 += U) {
         uint4 xv[G][U];
         uint4 av[RPG][U];
         bool cv[U];
@@ -164,18 +200,6 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll
             for (int i = 0; i < RPG; i++) av[i][u] = ap[i][cs];
         }
-        if constexpr (PF && !BT) {
-            if (first && pf_active) {
-#pragma unroll
-                for (int jj = 0; jj < EB; jj++) {
-                    const int row = __builtin_amdgcn_readfirstlane(s_brow[jj]);
-                    bpre[jj] = row >= 0 ? ldg16(brows + (size_t)row * hout + (size_t)tid * 8) : zero16();
-                }
-#pragma unroll
-                for (int k = 0; k < G; k++)
-                    ypre[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)tid * 8) : zero16();
-            }
-        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
 #pragma unroll
@@ -188,19 +212,30 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll
                 for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
         }
-    };
-    shrink_round(0, true);
-#pragma unroll 1
-    for (int it0 = U; it0 < n_it; it0 += U) shrink_round(it0, false);
+    }
+
+    // First expand step requested now: its latency runs under the reduction and the two barriers.
+    uint4 bpre[PF ? EB : 1];
+    uint4 ypre[PF ? G : 1];
+    if constexpr (PF) {
+        if (tid < ncc_out) {
+            int br[EB];
+            b_rows_of(0, br);
 #pragma unroll
-    for (int k = 0; k < G; k++)
+            for (int jj = 0; jj < EB; jj++)
+                bpre[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)tid * 8) : zero16();
 #pragma unroll
-        for (int i = 0; i < RPG; i++) acc[k][i] = ((row_ok >> i) & 1u) ? acc[k][i] : 0.f;
+            for (int k = 0; k < G; k++)
+                ypre[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)tid * 8) : zero16();
+        }
+    }
+
 #pragma unroll
     for (int k = 0; k < G; k++)
 #pragma unroll
         for (int i = 0; i < RPG; i++) {
-            const float s = row16_sum(acc[k][i]);
+            const float a = ((row_ok >> i) & 1u) ? acc[k][i] : 0.f;
+            const float s = row16_sum(a);
             if (cl == 0) s_part[wave][k][rg + 4 * i] = s;
         }
     __syncthreads();
@@ -223,7 +258,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             for (int k = 0; k < G; k++) {
                 if (p.accumulate && tok[k] >= 0) {
                     uint4 yv;
-                    if (PF && pre) yv = ypre[k]; else yv = ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8);
+                    if (pre) yv = ypre[k]; else yv = ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8);
                     unpack8<DT>(yv, o[k]);
                 } else {
 #pragma unroll
@@ -233,15 +268,15 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
 #pragma unroll 1
             for (int j0 = 0; j0 < r; j0 += EB) {
                 uint4 bv[EB];
-                if (PF && pre && j0 == 0) {
+                if (pre && j0 == 0) {
 #pragma unroll
                     for (int jj = 0; jj < EB; jj++) bv[jj] = bpre[jj];
                 } else {
+                    int br[EB];
+                    b_rows_of(j0, br);
 #pragma unroll
-                    for (int jj = 0; jj < EB; jj++) {
-                        const int row = __builtin_amdgcn_readfirstlane(s_brow[j0 + jj]);
-                        bv[jj] = row >= 0 ? ldg16(brows + (size_t)row * hout + (size_t)cc * 8) : zero16();
-                    }
+                    for (int jj = 0; jj < EB; jj++)
+                        bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
                 }
 #pragma unroll
                 for (int jj = 0; jj < EB; jj++) {
@@ -321,26 +356,27 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
     }
 }
 
-template <int DT, int G, int RMAX, int NT, bool BT, bool PF = false>
+template <int DT, int G, int RMAX, bool BT, bool WORK>
 static int launch_one(const BgmvArgs &a, hipStream_t s)
 {
-    const long long total = (long long)a.n_proj * a.items_per_proj;
-    const unsigned grid = (unsigned)(((total + 7) / 8) * 8);
-    if (grid == 0) return 0;
-    hipLaunchKernelGGL((bgmv_kernel<DT, G, RMAX, NT, BT, PF>), dim3(grid), dim3(NT), 0, s, a);
+    constexpr int NT = 256;
+    const long long per_proj = WORK ? a.work_cap : a.T;
+    const long long total = (long long)a.n_proj * per_proj;
+    if (total <= 0) return 0;
+    if (total > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((bgmv_kernel<DT, G, RMAX, NT, BT, WORK>), dim3((unsigned)total), dim3(NT), 0, s, a);
     return (int)hipGetLastError();
 }
 
-template <int DT, int RMAX, bool BT>
-static int launch_g(const BgmvArgs &a, int group, hipStream_t s)
+template <int DT, int RMAX>
+static int launch_work(const BgmvArgs &a, int group, hipStream_t s)
 {
-    constexpr int NT = 256;
     switch (group) {
-    case 1: return launch_one<DT, 1, RMAX, NT, BT>(a, s);
-    case 2: return launch_one<DT, 2, RMAX, NT, BT>(a, s);
-    case 4: return launch_one<DT, 4, RMAX, NT, BT>(a, s);
+    case 1: return launch_one<DT, 1, RMAX, false, true>(a, s);
+    case 2: return launch_one<DT, 2, RMAX, false, true>(a, s);
+    case 4: return launch_one<DT, 4, RMAX, false, true>(a, s);
     case 8:
-        if constexpr (RMAX <= 32) return launch_one<DT, 8, RMAX, NT, BT>(a, s);
+        if constexpr (RMAX <= 32) return launch_one<DT, 8, RMAX, false, true>(a, s);
         else return (int)hipErrorInvalidValue;
     default: return (int)hipErrorInvalidValue;
     }
@@ -349,16 +385,21 @@ static int launch_g(const BgmvArgs &a, int group, hipStream_t s)
 template <int DT>
 static int launch_dt(const BgmvArgs &a, int group, int max_rank, bool bt, hipStream_t s)
 {
-    if (bt) {
-        // the reference-layout call is one token per work item
-        if (group != 1) return (int)hipErrorInvalidValue;
-        if (max_rank <= 16) return launch_one<DT, 1, 16, 256, true>(a, s);
-        if (max_rank <= 32) return launch_one<DT, 1, 32, 256, true>(a, s);
-        return launch_one<DT, 1, 64, 256, true>(a, s);
+    if (a.work) {
+        if (bt) return (int)hipErrorInvalidValue;
+        if (max_rank <= 16) return launch_work<DT, 16>(a, group, s);
+        if (max_rank <= 32) return launch_work<DT, 32>(a, group, s);
+        return launch_work<DT, 64>(a, group, s);
     }
-    if (max_rank <= 16) return launch_g<DT, 16, false>(a, group, s);
-    if (max_rank <= 32) return launch_g<DT, 32, false>(a, group, s);
-    return launch_g<DT, 64, false>(a, group, s);
+    if (group != 1) return (int)hipErrorInvalidValue;      // the plain form is one token per work item
+    if (bt) {
+        if (max_rank <= 16) return launch_one<DT, 1, 16, true, false>(a, s);
+        if (max_rank <= 32) return launch_one<DT, 1, 32, true, false>(a, s);
+        return launch_one<DT, 1, 64, true, false>(a, s);
+    }
+    if (max_rank <= 16) return launch_one<DT, 1, 16, false, false>(a, s);
+    if (max_rank <= 32) return launch_one<DT, 1, 32, false, false>(a, s);
+    return launch_one<DT, 1, 64, false, false>(a, s);
 }
 
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s)

@@ -30,11 +30,12 @@ int log2_exact(int v)
     return -1;
 }
 
-int check_pool(mlora::PoolView &pv, const int32_t *a_tbl, const int32_t *b_tbl, const int32_t *rank,
-               const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages_a,
-               int64_t n_pages_b, int max_rank)
+int check_pool(mlora::PoolView &pv, const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+               int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank)
 {
-    if (!a_tbl || !b_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page tables, rank and scaling must not be NULL");
+    const int32_t *a_tbl = page_tbl, *b_tbl = page_tbl;
+    const int64_t n_pages_a = n_pages, n_pages_b = n_pages;
+    if (!page_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page table, rank and scaling must not be NULL");
     if (n_adapters <= 0) return fail(MLORA_EINVAL, "n_adapters must be positive (got %d)", n_adapters);
     const int shift = log2_exact(page_rows);
     if (shift < 0 || page_rows > 64) return fail(MLORA_EINVAL, "page_rows must be a power of two in 1..64 (got %d)", page_rows);
@@ -42,7 +43,7 @@ int check_pool(mlora::PoolView &pv, const int32_t *a_tbl, const int32_t *b_tbl, 
     if (max_rank < 1 || max_rank > MLORA_MAX_RANK) return fail(MLORA_ERANGE, "max_rank must be in 1..%d (got %d)", MLORA_MAX_RANK, max_rank);
     if ((int64_t)max_pages * page_rows < max_rank)
         return fail(MLORA_ERANGE, "max_pages * page_rows = %lld cannot hold max_rank %d", (long long)max_pages * page_rows, max_rank);
-    if (n_pages_a <= 0 || n_pages_b <= 0) return fail(MLORA_EINVAL, "n_pages_a / n_pages_b must be positive");
+    if (n_pages <= 0) return fail(MLORA_EINVAL, "n_pages must be positive");
     if (n_pages_a * page_rows > 0x7fffffffLL || n_pages_b * page_rows > 0x7fffffffLL)
         return fail(MLORA_ERANGE, "a rows slab may hold at most 2^31-1 rows");
     pv.a_tbl = a_tbl; pv.b_tbl = b_tbl; pv.rank = rank; pv.scaling = scaling;
@@ -68,10 +69,11 @@ const char *mlora_last_error(void) { return g_err; }
 int mlora_version(void) { return 100; }
 
 int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
-                      const float *scaling, int n_adapters, int max_pages, int page_rows,
+                      const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
                       int32_t *out_row_off, int32_t *out_rank, float *out_scale, int32_t *perm,
                       int32_t *seg_start, int32_t *seg_len, int32_t *seg_adapter, int32_t *chunk_start,
-                      int32_t *chunk_len, int32_t *chunk_adapter, int group, int32_t *counters, void *stream)
+                      int32_t *chunk_len, int32_t *chunk_adapter, int group, int32_t *counters, int32_t *work,
+                      void *stream)
 {
     if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
     if (T == 0) return MLORA_OK;
@@ -82,12 +84,17 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
         if (!page_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page_tbl, rank and scaling are needed for the per-token view");
         if (max_pages <= 0 || page_rows <= 0) return fail(MLORA_EINVAL, "max_pages and page_rows must be positive");
     }
-    const bool grouped = perm || seg_start || seg_len || seg_adapter || chunk_start || chunk_len || chunk_adapter || counters;
+    const bool grouped = perm || seg_start || seg_len || seg_adapter || chunk_start || chunk_len || chunk_adapter || counters || work;
     if (grouped) {
         if (!(perm && seg_start && seg_len && seg_adapter && chunk_start && chunk_len && chunk_adapter && counters))
             return fail(MLORA_EINVAL, "the grouped view needs all of perm, seg_*, chunk_* and counters");
         if (T > MLORA_GATHER_MAX_T) return fail(MLORA_ERANGE, "T = %d exceeds MLORA_GATHER_MAX_T = %d", T, MLORA_GATHER_MAX_T);
         if (group != 1 && group != 2 && group != 4 && group != 8) return fail(MLORA_EINVAL, "group must be 1, 2, 4 or 8 (got %d)", group);
+        if (work) {
+            if (!page_tbl || !rank || !scaling) return fail(MLORA_EINVAL, "page_tbl, rank and scaling are needed for the work records");
+            if (max_pages <= 0 || page_rows <= 0 || n_pages <= 0) return fail(MLORA_EINVAL, "max_pages, page_rows and n_pages must be positive");
+            if (n_pages * (int64_t)page_rows > 0x7fffffffLL) return fail(MLORA_ERANGE, "a rows slab may hold at most 2^31-1 rows");
+        }
     }
     if (!per_tok && !grouped) return MLORA_OK;
     mlora::GatherArgs a;
@@ -97,6 +104,7 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
     a.out_row_off = out_row_off; a.out_rank = out_rank; a.out_scale = out_scale;
     a.perm = perm; a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter;
     a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_adapter = chunk_adapter; a.counters = counters;
+    a.n_pages = n_pages; a.work = work; a.work_cap = MLORA_WORK_CAP(T);
     const int rc = mlora::launch_gather(a, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "gather launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
@@ -104,11 +112,9 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
 
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
                      const void *const *b_rows, const int32_t *hin, const int32_t *hout,
-                     const int32_t *tok_adapter, int T, const int32_t *a_page_tbl, const int32_t *b_page_tbl,
-                     const int32_t *rank, const float *scaling, int n_adapters, int max_pages, int page_rows,
-                     int64_t n_pages_a, int64_t n_pages_b, int max_rank, const int32_t *perm,
-                     const int32_t *chunk_start, const int32_t *chunk_len, const int32_t *chunk_adapter,
-                     const int32_t *counters, int group, int dtype, int accumulate, void *stream)
+                     const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
+                     const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
+                     int max_rank, const int32_t *work, int group, int dtype, int accumulate, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
@@ -118,16 +124,14 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
     if (!tok_adapter) return fail(MLORA_EINVAL, "tok_adapter must not be NULL");
     mlora::BgmvArgs a;
     memset(&a, 0, sizeof(a));
-    int rc = check_pool(a.pool, a_page_tbl, b_page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank);
+    int rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
     if (rc) return rc;
-    const bool grouped = perm != nullptr;
-    if (grouped) {
-        if (!(chunk_start && chunk_len && chunk_adapter && counters)) return fail(MLORA_EINVAL, "a grouped launch needs perm, chunk_* and counters");
+    if (work) {
         if (group != 1 && group != 2 && group != 4 && group != 8) return fail(MLORA_EINVAL, "group must be 1, 2, 4 or 8 (got %d)", group);
         if (group == 8 && max_rank > 32) return fail(MLORA_ERANGE, "group 8 supports max_rank <= 32 (got %d); use group 4", max_rank);
-    } else {
-        if (chunk_start || chunk_len || chunk_adapter) return fail(MLORA_EINVAL, "chunk arrays given without perm");
-        if (group != 1) return fail(MLORA_EINVAL, "group must be 1 when perm is NULL (got %d)", group);
+        if (!aligned16(work)) return fail(MLORA_EALIGN, "work records must be 16-byte aligned");
+    } else if (group != 1) {
+        return fail(MLORA_EINVAL, "group must be 1 when work is NULL (got %d)", group);
     }
     for (int p = 0; p < n_proj; p++) {
         if (!y[p] || !x[p] || !a_rows[p] || !b_rows[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
@@ -139,24 +143,23 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
         a.hin[p] = hin[p]; a.hout[p] = hout[p];
     }
     a.tok_adapter = tok_adapter; a.tok_adapter64 = nullptr;
-    a.perm = perm; a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_adapter = chunk_adapter; a.counters = counters;
-    a.T = T; a.n_proj = n_proj; a.items_per_proj = T; a.accumulate = accumulate ? 1 : 0;
+    a.work = work; a.work_cap = MLORA_WORK_CAP(T);
+    a.T = T; a.n_proj = n_proj; a.accumulate = accumulate ? 1 : 0;
     rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
 }
 
 int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *tok_adapter,
-               const int32_t *a_page_tbl, const int32_t *b_page_tbl, const int32_t *rank, const float *scaling,
-               int T, int hin, int hout, int n_adapters, int max_pages, int page_rows, int64_t n_pages_a,
-               int64_t n_pages_b, int max_rank, int dtype, int accumulate, void *stream)
+               const int32_t *page_tbl, const int32_t *rank, const float *scaling, int T, int hin, int hout,
+               int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank, int dtype,
+               int accumulate, void *stream)
 {
     void *ys[1] = {y};
     const void *xs[1] = {x}, *as[1] = {a_rows}, *bs[1] = {b_rows};
     const int32_t hi[1] = {hin}, ho[1] = {hout};
-    return mlora_bgmv_multi(1, ys, xs, as, bs, hi, ho, tok_adapter, T, a_page_tbl, b_page_tbl, rank, scaling,
-                            n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank, nullptr, nullptr,
-                            nullptr, nullptr, nullptr, 1, dtype, accumulate, stream);
+    return mlora_bgmv_multi(1, ys, xs, as, bs, hi, ho, tok_adapter, T, page_tbl, rank, scaling, n_adapters,
+                            max_pages, page_rows, n_pages, max_rank, nullptr, 1, dtype, accumulate, stream);
 }
 
 int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const void *wb_T_all,
@@ -194,7 +197,7 @@ int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const voi
         return fail(MLORA_EALIGN, "layer slab of the pool is not 16-byte aligned (r * hin and hout * r must be multiples of 8)");
     a.hin[0] = hin; a.hout[0] = hout;
     a.tok_adapter = nullptr; a.tok_adapter64 = indices;
-    a.T = T; a.n_proj = 1; a.items_per_proj = T; a.accumulate = 1;
+    a.T = T; a.n_proj = 1; a.accumulate = 1;
     rc = mlora::launch_bgmv(a, dtype, 1, r, true, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
@@ -249,9 +252,9 @@ int64_t mlora_sgmv_workspace_bytes(int T, int n_seg)
 }
 
 int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
-               const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *a_page_tbl,
-               const int32_t *b_page_tbl, const int32_t *rank, const float *scaling, int T, int hin, int hout,
-               int n_adapters, int max_pages, int page_rows, int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
+               const int32_t *rank, const float *scaling, int T, int hin, int hout,
+               int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
                int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
@@ -264,7 +267,7 @@ int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, c
         return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
     mlora::SgmvArgs a;
     memset(&a, 0, sizeof(a));
-    rc = check_pool(a.pool, a_page_tbl, b_page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages_a, n_pages_b, max_rank);
+    rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
     if (rc) return rc;
     const SgmvWs w = sgmv_layout(T, n_seg);
     if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");

@@ -8,6 +8,10 @@ namespace mlora {
 
 constexpr int MAX_PROJ = 8;
 constexpr int MAX_RANK = 64;
+// Decode work record (int32 words): [0] tokens in the item (0 = empty), [1] adapter (-1 = none),
+// [2] rank, [3] scaling (float bits), [4..11] token ids, [12..15] zero, [16..79] row of rank row j (-1 = absent).
+constexpr int WORK_WORDS = 80;
+constexpr int WORK_ROWS_AT = 16;
 
 // How the rank rows of an adapter are found inside a rows slab.
 struct PoolView {
@@ -36,14 +40,10 @@ struct BgmvArgs {
     PoolView pool;
     const int32_t *tok_adapter;    // [T] int32, or nullptr when tok_adapter64 is used
     const int64_t *tok_adapter64;  // [T] int64 (reference layout call)
-    const int32_t *perm;           // grouped view (nullptr => one token per work item)
-    const int32_t *chunk_start;
-    const int32_t *chunk_len;
-    const int32_t *chunk_adapter;
-    const int32_t *counters;
+    const int32_t *work;           // work records in launch order (nullptr => one token per workgroup)
+    int work_cap;                  // records (= workgroups per projection), a multiple of 8
     int T;
     int n_proj;
-    int items_per_proj;            // work-item bound per projection (T)
     int accumulate;
 };
 
@@ -53,6 +53,9 @@ struct GatherArgs {
     const int32_t *rank;
     const float *scaling;
     int T, n_adapters, max_pages, page_rows, group;
+    long long n_pages;             // pages in a rows slab (bounds the recorded rows)
+    int32_t *work;                 // [work_cap * WORK_WORDS] decode work records, or nullptr
+    int work_cap;
     int32_t *out_row_off;
     int32_t *out_rank;
     float *out_scale;

@@ -198,6 +198,41 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
             ch_idx++;
         }
     }
+    // ---- decode work records, in launch order: workgroup b of a projection reads record b.
+    // Consecutive chunks go to the same XCD (workgroups are dealt to the 8 XCDs round-robin).
+    if (g.work) {
+        __shared__ int s_nchunks;
+        if (tid == GATHER_NT - 1) s_nchunks = ch_incl;
+        __syncthreads();                         // chunk_* arrays written above are visible to the whole block
+        const int n_chunks = s_nchunks;
+        const int per_xcd = (n_chunks + 7) >> 3;
+        const long long words = (long long)g.work_cap * WORK_WORDS;
+        for (long long idx = tid; idx < words; idx += GATHER_NT) {
+            const int b = (int)(idx / WORK_WORDS), w = (int)(idx - (long long)b * WORK_WORDS);
+            const int c = (b & 7) * per_xcd + (b >> 3);
+            int val = w == 1 ? -1 : 0;
+            if ((b >> 3) < per_xcd && c < n_chunks) {
+                const int start = g.chunk_start[c], len = g.chunk_len[c], a = g.chunk_adapter[c];
+                int rk = 0;
+                if (a >= 0) { rk = g.rank[a]; rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); }
+                if (w == 0) val = len;
+                else if (w == 1) val = a;
+                else if (w == 2) val = rk;
+                else if (w == 3) val = a >= 0 ? __builtin_bit_cast(int, g.scaling[a]) : 0;
+                else if (w < 12) val = (w - 4) < len ? (int)(s_key[start + (w - 4)] & ((1u << TOK_BITS) - 1u)) : -1;
+                else if (w < WORK_ROWS_AT) val = 0;
+                else {
+                    const int j = w - WORK_ROWS_AT;
+                    val = -1;
+                    if (a >= 0 && j < rk && j / g.page_rows < g.max_pages) {
+                        const int pg = g.page_tbl[(long long)a * g.max_pages + j / g.page_rows];
+                        if (pg >= 0 && pg < g.n_pages) val = pg * g.page_rows + j % g.page_rows;
+                    }
+                }
+            }
+            g.work[idx] = val;
+        }
+    }
     if (tid == GATHER_NT - 1) {
         g.counters[0] = seg_incl;
         g.counters[1] = n_valid;

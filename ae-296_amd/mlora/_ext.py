@@ -22,6 +22,12 @@ MAX_PROJ = 8
 MAX_RANK = 64
 GATHER_MAX_T = 8192
 CNT_NSEG, CNT_NVALID, CNT_NCHUNK, CNT_BAD, CNT_WORDS = 0, 1, 2, 3, 8
+WORK_WORDS = 80
+
+
+def work_cap(T: int) -> int:
+    return ((T + 7) // 8) * 8
+
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 
@@ -29,16 +35,16 @@ _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
 SIGNATURES = {
     "mlora_last_error": (C.c_char_p, []),
     "mlora_version": (_i32, []),
-    "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-                                 _vp, _vp, _vp, _i32, _vp, _vp]),
-    "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32,
-                                _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _vp]),
-    "mlora_bgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i64, _i64,
+    "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                 _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+    "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
+                                _i64, _i32, _vp, _i32, _i32, _i32, _vp]),
+    "mlora_bgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i64,
                           _i32, _i32, _i32, _vp]),
     "mlora_bgmv_reflayout": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
     "mlora_sgmv_workspace_bytes": (_i64, [_i32, _i32]),
-    "mlora_sgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
-                          _i32, _i64, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
+    "mlora_sgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
+                          _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     "mlora_prefill_reflayout": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _vp]),
 }
 

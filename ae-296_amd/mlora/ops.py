@@ -53,6 +53,7 @@ class DecodePlan:
     chunk_len: torch.Tensor
     chunk_adapter: torch.Tensor
     counters: torch.Tensor         # int32 [8]: n_seg, n_valid, n_chunks, n_bad
+    work: torch.Tensor             # int32 [work_cap(T), 80] decode work records in launch order
     row_off: Optional[torch.Tensor] = None   # int32 [T, max_pages]
     tok_rank: Optional[torch.Tensor] = None
     tok_scale: Optional[torch.Tensor] = None
@@ -80,7 +81,8 @@ def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: int = 4, pe
         out = DecodePlan(tok_adapter, group, torch.empty(max(T, 1), **i32), torch.empty(nseg, **i32),
                          torch.empty(nseg, **i32), torch.empty(nseg, **i32), torch.empty(max(T, 1), **i32),
                          torch.empty(max(T, 1), **i32), torch.empty(max(T, 1), **i32),
-                         torch.zeros(_ext.CNT_WORDS, **i32))
+                         torch.zeros(_ext.CNT_WORDS, **i32),
+                         torch.empty((max(_ext.work_cap(T), 8), _ext.WORK_WORDS), **i32))
         if per_token:
             out.row_off = torch.empty((max(T, 1), pool.max_pages), **i32)
             out.tok_rank = torch.empty(max(T, 1), **i32)
@@ -90,11 +92,11 @@ def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: int = 4, pe
         out.group = group
     rc = _ext.lib().mlora_pool_gather(
         _ext.ptr(tok_adapter), T, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
-        pool.n_slots, pool.max_pages, pool.page_rows,
+        pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages,
         _ext.ptr(out.row_off), _ext.ptr(out.tok_rank), _ext.ptr(out.tok_scale),
         _ext.ptr(out.perm), _ext.ptr(out.seg_start), _ext.ptr(out.seg_len), _ext.ptr(out.seg_adapter),
         _ext.ptr(out.chunk_start), _ext.ptr(out.chunk_len), _ext.ptr(out.chunk_adapter), group,
-        _ext.ptr(out.counters), _ext.current_stream_ptr())
+        _ext.ptr(out.counters), _ext.ptr(out.work), _ext.current_stream_ptr())
     _ext.check(rc)
     return out
 
@@ -126,14 +128,11 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     pool.sync()
     if plan is not None and plan.T != T:
         raise ValueError("plan was built for a different batch size")
-    pp = plan
     rc = _ext.lib().mlora_bgmv_multi(
         n, yv, xv, av, bv, hi, ho, _ext.ptr(tok_adapter), T,
-        _ext.ptr(pool.page_tbl), _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
-        pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.n_pages, pool.max_rank,
-        _ext.ptr(pp.perm) if pp else None, _ext.ptr(pp.chunk_start) if pp else None,
-        _ext.ptr(pp.chunk_len) if pp else None, _ext.ptr(pp.chunk_adapter) if pp else None,
-        _ext.ptr(pp.counters) if pp else None, pp.group if pp else 1,
+        _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
+        pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.max_rank,
+        _ext.ptr(plan.work) if plan else None, plan.group if plan else 1,
         pool.dtype_code, int(accumulate), _ext.current_stream_ptr())
     _ext.check(rc)
 
@@ -196,8 +195,8 @@ def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: 
     a_ptr, b_ptr = pool.slab_ptrs(layer, proj)
     rc = _ext.lib().mlora_sgmv(
         y.data_ptr(), x.data_ptr(), a_ptr, b_ptr, seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(),
-        n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
-        T, hin, hout, pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.n_pages, pool.max_rank,
+        n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
+        T, hin, hout, pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.max_rank,
         pool.dtype_code, int(accumulate), workspace.data_ptr(), workspace.numel(), _ext.current_stream_ptr())
     _ext.check(rc)
 

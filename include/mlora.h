@@ -29,9 +29,9 @@
  *               base 16-byte aligned.  An A slab holds rank rows of A^T (length Hin),
  *               a B slab holds rank rows of B (length Hout).
  *   page_tbl  : int32 [n_adapters, max_pages]; rank row j of adapter i is row
- *               page_tbl[i][j / page_rows] * page_rows + j % page_rows.
- *               page_rows is a power of two (1..64).  A NULL page table means the
- *               dense layout: rank row j of adapter i is row i * dense_stride_rows + j.
+ *               page_tbl[i][j / page_rows] * page_rows + j % page_rows, in the A slab and in the
+ *               B slab alike (one table serves every layer, projection and side).
+ *               page_rows is a power of two (1..64).
  *   rank      : int32 [n_adapters], 1..max_rank (max_rank <= 64).
  *   scaling   : float [n_adapters]  (alpha / r).
  *   tok_adapter : int32 [T]; a negative value means the token has no adapter.
@@ -67,6 +67,11 @@ extern "C" {
 #define MLORA_CNT_BAD 3      /* tokens whose adapter id was >= n_adapters (treated as none) */
 #define MLORA_CNT_WORDS 8
 
+/* Decode work records written by mlora_pool_gather and read by mlora_bgmv_multi: one record of
+ * MLORA_WORK_WORDS int32 per workgroup and projection, MLORA_WORK_CAP(T) records per batch. */
+#define MLORA_WORK_WORDS 80
+#define MLORA_WORK_CAP(T) ((((T) + 7) / 8) * 8)
+
 const char *mlora_last_error(void);
 int mlora_version(void);
 
@@ -84,15 +89,21 @@ int mlora_version(void);
  *   chunk_start/len/adapter [T]   each segment cut into pieces of <= group tokens, then the
  *                       adapter-less tokens in pieces of <= group with adapter -1
  *   counters [MLORA_CNT_WORDS]
+ *   work [MLORA_WORK_CAP(T) * MLORA_WORK_WORDS]  (optional, may be NULL) the chunks as decode work
+ *                       records in launch order: chunk c is record (c mod P) * 8 + c / P with
+ *                       P = ceil(n_chunks / 8), so consecutive chunks run on one XCD.  Record words:
+ *                       [0] tokens (0 = empty record) [1] adapter [2] rank [3] scaling (float bits)
+ *                       [4..11] token ids [12..15] 0 [16..79] row of rank row j in a rows slab, -1 if
+ *                       j >= rank or the page id is outside [0, n_pages).
  * T <= MLORA_GATHER_MAX_T.  All outputs are exact integers / copied floats (bit-exact).
  */
 int mlora_pool_gather(const int32_t *tok_adapter, int T,
                       const int32_t *page_tbl, const int32_t *rank, const float *scaling,
-                      int n_adapters, int max_pages, int page_rows,
+                      int n_adapters, int max_pages, int page_rows, int64_t n_pages,
                       int32_t *out_row_off, int32_t *out_rank, float *out_scale,
                       int32_t *perm, int32_t *seg_start, int32_t *seg_len, int32_t *seg_adapter,
                       int32_t *chunk_start, int32_t *chunk_len, int32_t *chunk_adapter, int group,
-                      int32_t *counters, void *stream);
+                      int32_t *counters, int32_t *work, void *stream);
 
 /*
  * Decode (BGMV): for every token t with adapter a = tok_adapter[t] and every projection p
@@ -104,32 +115,28 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T,
  *
  * y, x, a_rows, b_rows, hin, hout are HOST arrays of n_proj entries (device pointers /
  * sizes per projection; projections may share x).  x_p is [T, hin[p]], y_p is [T, hout[p]].
- * The page tables, rank and scaling are shared by all projections of the call.
- * n_pages_a / n_pages_b bound the page ids (rows slab extents) for in-kernel checks.
- * Grouped launch: pass the perm / chunk_* / counters arrays written by
- * mlora_pool_gather with the same `group` (1, 2, 4 or 8) and max_chunks = T; tokens of one
- * adapter then share one read of its rows.  With perm == NULL every token is its own
- * work item and group must be 1.
+ * The page table, rank and scaling are shared by all projections of the call; n_pages bounds the
+ * page ids (rows slab extent) for in-kernel checks.
+ * Grouped launch: pass the `work` records written by mlora_pool_gather for this batch with the
+ * same `group` (1, 2, 4 or 8; 8 needs max_rank <= 32); tokens of one adapter then share one read
+ * of its rows and each workgroup starts from one record instead of walking the tables.
+ * With work == NULL every token is its own work item and group must be 1.
  */
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
                      const void *const *a_rows, const void *const *b_rows,
                      const int32_t *hin, const int32_t *hout,
                      const int32_t *tok_adapter, int T,
-                     const int32_t *a_page_tbl, const int32_t *b_page_tbl,
-                     const int32_t *rank, const float *scaling,
-                     int n_adapters, int max_pages, int page_rows,
-                     int64_t n_pages_a, int64_t n_pages_b, int max_rank,
-                     const int32_t *perm, const int32_t *chunk_start, const int32_t *chunk_len,
-                     const int32_t *chunk_adapter, const int32_t *counters, int group,
+                     const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                     int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                     const int32_t *work, int group,
                      int dtype, int accumulate, void *stream);
 
 /* One projection, one token per work item: the plain form of the call above. */
 int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
                const int32_t *tok_adapter,
-               const int32_t *a_page_tbl, const int32_t *b_page_tbl,
-               const int32_t *rank, const float *scaling,
+               const int32_t *page_tbl, const int32_t *rank, const float *scaling,
                int T, int hin, int hout, int n_adapters, int max_pages, int page_rows,
-               int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               int64_t n_pages, int max_rank,
                int dtype, int accumulate, void *stream);
 
 /*
@@ -157,10 +164,9 @@ int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const voi
 int64_t mlora_sgmv_workspace_bytes(int T, int n_seg);
 int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
                const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
-               const int32_t *a_page_tbl, const int32_t *b_page_tbl,
-               const int32_t *rank, const float *scaling,
+               const int32_t *page_tbl, const int32_t *rank, const float *scaling,
                int T, int hin, int hout, int n_adapters, int max_pages, int page_rows,
-               int64_t n_pages_a, int64_t n_pages_b, int max_rank,
+               int64_t n_pages, int max_rank,
                int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*

@@ -18,7 +18,7 @@
  *
  * Pinned functions (see tests/test_oracle_*.py):
  *   orc_f16_to_f32 / orc_f32_to_f16 / orc_bf16_* : exhaustive / randomized vs numpy & torch
- *   orc_pool_gather, orc_build_segments, orc_build_chunks, orc_sgmv_plan : vs numpy closed forms
+ *   orc_pool_gather, orc_build_segments, orc_build_chunks, orc_build_work, orc_sgmv_plan : vs numpy closed forms / enumeration
  *   orc_lora_apply_paged      : brute-force fp64 loops, one-hot, scale 0, library matmul
  *   orc_add_lora_bgmv_ref     : same expression through numpy on the reference layout
  *   orc_prefill_bmm_ref       : numpy matmul pairs (the reference's bmm.bmm)
@@ -208,6 +208,50 @@ int orc_build_chunks(const int32_t *seg_start, const int32_t *seg_len, const int
         nc++;
     }
     *n_chunks = nc;
+    return ORC_OK;
+}
+
+/* Decode work records for the fused decode kernel, in launch order.  Chunk c is served by the
+ * workgroup b = (c mod per_xcd) * 8 + c / per_xcd with per_xcd = ceil(n_chunks / 8): workgroups are
+ * dealt to the 8 XCDs round-robin by id, so consecutive chunks land on one XCD.  Record b
+ * (ORC_WORK_WORDS int32): [0] tokens in the chunk (0 = empty record), [1] adapter (-1 = none),
+ * [2] rank clamped to 0..64, [3] scaling as float bits, [4..11] token ids (-1 unused), [12..15] 0,
+ * [16..79] row of rank row j = page_tbl[a][j / page_rows] * page_rows + j % page_rows, or -1 when
+ * j >= rank or the page id is outside [0, n_pages).  This is layout bookkeeping of this build (the
+ * reference has no counterpart); it is pinned by direct enumeration in the tests. */
+#define ORC_WORK_WORDS 80
+int orc_build_work(const int32_t *chunk_start, const int32_t *chunk_len, const int32_t *chunk_adapter,
+                   int n_chunks, const int32_t *perm, const int32_t *page_tbl, const int32_t *rank,
+                   const float *scaling, int max_pages, int page_rows, int64_t n_pages,
+                   int work_cap, int32_t *work /* [work_cap * ORC_WORK_WORDS] */)
+{
+    if (work_cap < 0 || (work_cap & 7) || n_chunks > work_cap) return ORC_EINVAL;
+    int per_xcd = (n_chunks + 7) / 8;
+    for (int b = 0; b < work_cap; b++) {
+        int32_t *w = work + (size_t)b * ORC_WORK_WORDS;
+        for (int i = 0; i < ORC_WORK_WORDS; i++) w[i] = 0;
+        w[1] = -1;
+    }
+    for (int c = 0; c < n_chunks; c++) {
+        int b = (c % per_xcd) * 8 + c / per_xcd;
+        int32_t *w = work + (size_t)b * ORC_WORK_WORDS;
+        int a = chunk_adapter[c];
+        int rk = 0;
+        if (a >= 0) { rk = rank[a]; if (rk < 0) rk = 0; if (rk > 64) rk = 64; }
+        w[0] = chunk_len[c];
+        w[1] = a;
+        w[2] = rk;
+        if (a >= 0) memcpy(&w[3], &scaling[a], 4);
+        for (int k = 0; k < 8; k++) w[4 + k] = k < chunk_len[c] ? perm[chunk_start[c] + k] : -1;
+        for (int j = 0; j < 64; j++) {
+            int32_t v = -1;
+            if (a >= 0 && j < rk && j / page_rows < max_pages) {
+                int32_t pg = page_tbl[(size_t)a * max_pages + j / page_rows];
+                if (pg >= 0 && pg < n_pages) v = pg * page_rows + j % page_rows;
+            }
+            w[16 + j] = v;
+        }
+    }
     return ORC_OK;
 }
 

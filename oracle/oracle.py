@@ -123,6 +123,29 @@ def build_chunks(seg_start, seg_len, seg_adapter, n_valid, T, group):
     return cs[:n].copy(), cl[:n].copy(), ca[:n].copy()
 
 
+WORK_WORDS = 80
+
+
+def work_cap(T):
+    return ((T + 7) // 8) * 8
+
+
+def build_work(chunk_start, chunk_len, chunk_adapter, perm, page_tbl, rank, scaling, page_rows, n_pages, T):
+    cs = np.ascontiguousarray(chunk_start, np.int32)
+    cl = np.ascontiguousarray(chunk_len, np.int32)
+    ca = np.ascontiguousarray(chunk_adapter, np.int32)
+    perm = np.ascontiguousarray(perm, np.int32)
+    page_tbl = np.ascontiguousarray(page_tbl, np.int32)
+    rank = np.ascontiguousarray(rank, np.int32)
+    scaling = np.ascontiguousarray(scaling, np.float32)
+    cap = work_cap(T)
+    work = np.empty((cap, WORK_WORDS), np.int32)
+    rc = lib().orc_build_work(_p(cs), _p(cl), _p(ca), cs.size, _p(perm), _p(page_tbl), _p(rank), _p(scaling),
+                              page_tbl.shape[1], page_rows, C.c_int64(n_pages), cap, _p(work))
+    _check(rc, "build_work")
+    return work
+
+
 def sgmv_plan(seg_start, seg_len, tile):
     seg_start = np.ascontiguousarray(seg_start, np.int32)
     seg_len = np.ascontiguousarray(seg_len, np.int32)

@@ -48,7 +48,8 @@ def gather_case(seed, T, N, group, page_rows):
     perm, ss, sl, sa, nv = orc.build_segments(tok, N)
     cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, T, group)
     ro, rk, sc = orc.pool_gather(tok, page_tbl, rank, scaling, page_rows)
-    return dict(tok=tok, page_tbl=page_tbl, rank=rank, scaling=scaling, page_rows=page_rows, group=group, n_pages=nxt,
+    work = orc.build_work(cs, cl, ca, perm, page_tbl, rank, scaling, page_rows, nxt, T)
+    return dict(work=work, tok=tok, page_tbl=page_tbl, rank=rank, scaling=scaling, page_rows=page_rows, group=group, n_pages=nxt,
                 perm=perm, seg_start=ss, seg_len=sl, seg_adapter=sa, n_valid=nv, chunk_start=cs, chunk_len=cl,
                 chunk_adapter=ca, row_off=ro, tok_rank=rk, tok_scale=sc)
 

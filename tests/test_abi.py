@@ -42,12 +42,12 @@ def test_validation_errors_without_gpu():
     H = (C.c_int32 * 8)(64, 64, 64, 64, 64, 64, 64, 64)
 
     def bgmv(**kw):
-        a = dict(n_proj=1, hin=H, T=4, n_adapters=4, max_pages=8, page_rows=8, npa=10, npb=10, max_rank=64, perm=None,
+        a = dict(n_proj=1, hin=H, T=4, n_adapters=4, max_pages=8, page_rows=8, n_pages=10, max_rank=64, work=None,
                  group=1, dtype=0, y=P)
         a.update(kw)
-        return lib.mlora_bgmv_multi(a["n_proj"], a["y"], P, P, P, a["hin"], H, one, a["T"], one, one, one, one,
-                                    a["n_adapters"], a["max_pages"], a["page_rows"], a["npa"], a["npb"], a["max_rank"],
-                                    a["perm"], None, None, None, None, a["group"], a["dtype"], 1, None)
+        return lib.mlora_bgmv_multi(a["n_proj"], a["y"], P, P, P, a["hin"], H, one, a["T"], one, one, one,
+                                    a["n_adapters"], a["max_pages"], a["page_rows"], a["n_pages"], a["max_rank"],
+                                    a["work"], a["group"], a["dtype"], 1, None)
 
     assert bgmv(T=0) == _ext.MLORA_OK
     assert bgmv(dtype=7) == _ext.MLORA_EDTYPE
@@ -58,21 +58,25 @@ def test_validation_errors_without_gpu():
     assert bgmv(max_pages=1, page_rows=8, max_rank=16) == _ext.MLORA_ERANGE
     assert bgmv(hin=(C.c_int32 * 8)(60, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
     assert bgmv(y=(C.c_void_p * 8)(8, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
-    assert bgmv(group=4) == _ext.MLORA_EINVAL          # grouped launch without the grouped view
+    assert bgmv(group=4) == _ext.MLORA_EINVAL          # grouped launch without work records
+    assert bgmv(group=8, work=one, max_rank=64) == _ext.MLORA_ERANGE
+    assert bgmv(group=3, work=one) == _ext.MLORA_EINVAL
     assert bgmv(T=-1) == _ext.MLORA_EINVAL
     with pytest.raises(_ext.MloraError) as e:
         _ext.check(bgmv(dtype=7))
     assert e.value.code == _ext.MLORA_EDTYPE
 
-    rc = lib.mlora_pool_gather(one, 9000, one, one, one, 4, 8, 8, None, None, None, one, one, one, one, one, one, one, 4, one, None)
+    rc = lib.mlora_pool_gather(one, 9000, one, one, one, 4, 8, 8, 10, None, None, None, one, one, one, one, one, one, one, 4, one, one, None)
     assert rc == _ext.MLORA_ERANGE                     # more tokens than one gather call groups
-    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, None, None, None, one, None, one, one, one, one, one, 4, one, None)
+    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, 10, None, None, None, one, None, one, one, one, one, one, 4, one, None, None)
     assert rc == _ext.MLORA_EINVAL                     # incomplete grouped view
-    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, None, None, None, one, one, one, one, one, one, one, 3, one, None)
+    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, 10, None, None, None, one, one, one, one, one, one, one, 3, one, None, None)
     assert rc == _ext.MLORA_EINVAL                     # group not a power of two
+    rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, 0, None, None, None, one, one, one, one, one, one, one, 4, one, one, None)
+    assert rc == _ext.MLORA_EINVAL                     # work records need the slab extent
 
     assert lib.mlora_sgmv_workspace_bytes(9089, 16) > 9089 * 64 * 4
-    rc = lib.mlora_sgmv(one, one, one, one, one, one, one, 2, one, one, one, one, 100, 64, 64, 4, 8, 8, 10, 10, 64, 1, 1,
+    rc = lib.mlora_sgmv(one, one, one, one, one, one, one, 2, one, one, one, 100, 64, 64, 4, 8, 8, 10, 64, 1, 1,
                         one, 16, None)
     assert rc == _ext.MLORA_ENOSPACE
     rc = lib.mlora_bgmv_reflayout(one, one, one, one, one, 4, 8, 32, 16, 64, 64, 32, 1.0, 0, None)

@@ -29,6 +29,9 @@ def test_oracle_reproduces_gather():
     perm, ss, sl, sa, nv = orc.build_segments(d["tok"], N)
     cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, len(d["tok"]), int(d["group"]))
     ro, rk, sc = orc.pool_gather(d["tok"], d["page_tbl"], d["rank"], d["scaling"], int(d["page_rows"]))
+    work = orc.build_work(cs, cl, ca, perm, d["page_tbl"], d["rank"], d["scaling"], int(d["page_rows"]), int(d["n_pages"]),
+                          len(d["tok"]))
+    assert np.array_equal(work, d["work"])
     for got, key in ((perm, "perm"), (ss, "seg_start"), (sl, "seg_len"), (sa, "seg_adapter"), (cs, "chunk_start"),
                      (cl, "chunk_len"), (ca, "chunk_adapter"), (ro, "row_off"), (rk, "tok_rank")):
         assert np.array_equal(got, d[key]), key
@@ -110,6 +113,7 @@ def test_gpu_gather_meets_golden():
                         (plan.row_off, "row_off", None), (plan.tok_rank, "tok_rank", None)):
         assert np.array_equal(got.cpu().numpy()[:n], d[key]), key
     assert np.array_equal(plan.tok_scale.cpu().numpy().view(np.uint32), d["tok_scale"].view(np.uint32))
+    assert np.array_equal(plan.work.cpu().numpy(), d["work"])
 
 
 @pytest.mark.gpu

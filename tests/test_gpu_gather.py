@@ -43,6 +43,9 @@ def _check(tok, pool, group, n_bad_expected=0):
     assert np.array_equal(plan.chunk_start.cpu().numpy()[:n], cs)
     assert np.array_equal(plan.chunk_len.cpu().numpy()[:n], cl)
     assert np.array_equal(plan.chunk_adapter.cpu().numpy()[:n], ca)
+    want_work = orc.build_work(cs, cl, ca, perm, pool.h_page_tbl, pool.h_rank, pool.h_scaling, pool.page_rows,
+                               pool.n_pages, T)
+    assert np.array_equal(plan.work.cpu().numpy()[:want_work.shape[0]], want_work)
     assert np.array_equal(plan.row_off.cpu().numpy()[:T], ro)
     assert np.array_equal(plan.tok_rank.cpu().numpy()[:T], rk)
     assert np.array_equal(plan.tok_scale.cpu().numpy()[:T].view(np.uint32), sc.view(np.uint32))
@@ -87,9 +90,9 @@ def test_gather_reuses_buffers_and_is_idempotent():
     torch.cuda.synchronize()
     n = int(plan.counters[_ext.CNT_NCHUNK])
     first = [plan.perm.clone(), plan.chunk_start[:n].clone(), plan.chunk_len[:n].clone(),
-             plan.chunk_adapter[:n].clone(), plan.counters.clone()]
+             plan.chunk_adapter[:n].clone(), plan.counters.clone(), plan.work.clone()]
     plan_decode(tok, pool, group=4, out=plan)
     torch.cuda.synchronize()
-    second = [plan.perm, plan.chunk_start[:n], plan.chunk_len[:n], plan.chunk_adapter[:n], plan.counters]
+    second = [plan.perm, plan.chunk_start[:n], plan.chunk_len[:n], plan.chunk_adapter[:n], plan.counters, plan.work]
     for a, b in zip(first, second):
         assert torch.equal(a, b)

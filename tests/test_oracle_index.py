@@ -92,6 +92,45 @@ def test_build_chunks_brute_force(toks, group):
     assert len(cs) <= max(T, 1)
 
 
+def test_build_work_by_enumeration():
+    """Work records: placement b = (c mod P) * 8 + c // P and contents, checked field by field."""
+    rng = np.random.default_rng(8)
+    N, T, group, page_rows, n_pages = 9, 45, 4, 8, 40
+    rank = rng.choice([8, 16, 24, 64], N).astype(np.int32)
+    page_tbl = rng.integers(0, n_pages, (N, 8)).astype(np.int32)
+    page_tbl[3, 1] = n_pages + 5                  # a page id outside the slab -> rows marked absent
+    scaling = rng.random(N).astype(np.float32)
+    tok = rng.integers(-1, N, T).astype(np.int32)
+    perm, ss, sl, sa, nv = orc.build_segments(tok, N)
+    cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, T, group)
+    work = orc.build_work(cs, cl, ca, perm, page_tbl, rank, scaling, page_rows, n_pages, T)
+    cap = ((T + 7) // 8) * 8
+    assert work.shape == (cap, orc.WORK_WORDS)
+    P = -(-len(cs) // 8)
+    used = set()
+    for c in range(len(cs)):
+        b = (c % P) * 8 + c // P
+        used.add(b)
+        w = work[b]
+        a = int(ca[c])
+        assert w[0] == cl[c] and w[1] == a
+        assert w[4:4 + cl[c]].tolist() == perm[cs[c]:cs[c] + cl[c]].tolist() and np.all(w[4 + cl[c]:12] == -1)
+        assert np.all(w[12:16] == 0)
+        if a < 0:
+            assert w[2] == 0 and w[3] == 0 and np.all(w[16:] == -1)
+            continue
+        assert w[2] == rank[a] and w[3] == scaling[a:a + 1].view(np.int32)[0]
+        for j in range(64):
+            pg = page_tbl[a, j // page_rows]
+            want = pg * page_rows + j % page_rows if (j < rank[a] and 0 <= pg < n_pages) else -1
+            assert w[16 + j] == want
+    # consecutive chunks share blockIdx mod 8 (one XCD): chunk c sits at residue c // P
+    assert all(((c % P) * 8 + c // P) % 8 == c // P for c in range(len(cs)))
+    for b in range(cap):
+        if b not in used:
+            assert work[b, 0] == 0 and work[b, 1] == -1 and np.all(work[b, 2:] == 0)
+
+
 def test_sgmv_plan_brute_force():
     rng = np.random.default_rng(5)
     lens = rng.integers(0, 400, 23)
