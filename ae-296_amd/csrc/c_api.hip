@@ -209,15 +209,18 @@ namespace {
 
 constexpr int SG_TM = 64;   // tokens per tile, as in sgmv_prefill.hip
 
-struct SgmvWs { int max_tiles; int ksplit; size_t off_v, off_hi, off_lo, total; };
+struct SgmvWs { int max_tiles; int ksplit; size_t off_rec, off_v, off_hi, off_lo, total; };
 
 SgmvWs sgmv_layout(int T, int n_seg)
 {
     SgmvWs w;
     w.max_tiles = T / SG_TM + n_seg + 1;
-    int ks = (1024 + w.max_tiles - 1) / w.max_tiles;
+    int ks = (768 + w.max_tiles - 1) / w.max_tiles;      // about three shrink workgroups per CU
     w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : ks);
     size_t off = ((size_t)w.max_tiles * 3 + 4) * sizeof(int32_t);
+    off = (off + 255) & ~(size_t)255;
+    w.off_rec = off;
+    off += (size_t)w.max_tiles * 80 * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
     w.off_v = off;
     off += (size_t)w.ksplit * T * MLORA_MAX_RANK * sizeof(float);
@@ -235,6 +238,7 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
     int32_t *ip = reinterpret_cast<int32_t *>(base);
     a.tile_seg = ip; a.tile_tok0 = ip + w.max_tiles; a.tile_ntok = ip + 2 * (size_t)w.max_tiles;
     a.n_tiles = ip + 3 * (size_t)w.max_tiles;
+    a.tile_rec = reinterpret_cast<int32_t *>(base + w.off_rec);
     a.v = reinterpret_cast<float *>(base + w.off_v);
     a.vhi = reinterpret_cast<uint16_t *>(base + w.off_hi);
     a.vlo = reinterpret_cast<uint16_t *>(base + w.off_lo);
@@ -251,24 +255,27 @@ int64_t mlora_sgmv_workspace_bytes(int T, int n_seg)
     return (int64_t)sgmv_layout(T, n_seg).total;
 }
 
-int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
-               const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
-               const int32_t *rank, const float *scaling, int T, int hin, int hout,
-               int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
-               int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+static int sgmv_common(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
+                       const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
+                       const int32_t *rank, const float *scaling, int T, int hin, int hout, int n_adapters,
+                       int max_pages, int page_rows, int64_t n_pages, int max_rank, int dtype, int accumulate,
+                       void *workspace, int64_t workspace_bytes, int phases, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (T < 0 || n_seg < 0) return fail(MLORA_EINVAL, "T and n_seg must be >= 0 (got %d, %d)", T, n_seg);
     if (T == 0 || n_seg == 0) return MLORA_OK;
-    if (!y || !x || !a_rows || !b_rows || !seg_start || !seg_len || !seg_adapter) return fail(MLORA_EINVAL, "NULL device pointer");
-    int rc = check_dims(hin, hout);
-    if (rc) return rc;
-    if (!aligned16(y) || !aligned16(x) || !aligned16(a_rows) || !aligned16(b_rows))
-        return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+    if (!seg_start || !seg_len || !seg_adapter) return fail(MLORA_EINVAL, "NULL device pointer");
     mlora::SgmvArgs a;
     memset(&a, 0, sizeof(a));
-    rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
+    int rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
     if (rc) return rc;
+    if (phases & mlora::SGMV_APPLY) {
+        if (!y || !x || !a_rows || !b_rows) return fail(MLORA_EINVAL, "NULL device pointer");
+        rc = check_dims(hin, hout);
+        if (rc) return rc;
+        if (!aligned16(y) || !aligned16(x) || !aligned16(a_rows) || !aligned16(b_rows))
+            return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+    }
     const SgmvWs w = sgmv_layout(T, n_seg);
     if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
     if (workspace_bytes < (int64_t)w.total)
@@ -277,9 +284,41 @@ int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, c
     a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter; a.n_seg = n_seg;
     a.T = T; a.hin = hin; a.hout = hout; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0;
     carve(a, workspace, w);
-    rc = mlora::launch_sgmv(a, dtype, max_rank, static_cast<hipStream_t>(stream));
+    rc = mlora::launch_sgmv(a, dtype, max_rank, phases, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "sgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
+}
+
+int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
+               const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
+               const int32_t *rank, const float *scaling, int T, int hin, int hout,
+               int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+               int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return sgmv_common(y, x, a_rows, b_rows, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T, hin,
+                       hout, n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
+                       workspace_bytes, mlora::SGMV_PLAN | mlora::SGMV_APPLY, stream);
+}
+
+int mlora_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                    const int32_t *page_tbl, const int32_t *rank, const float *scaling, int T, int n_adapters,
+                    int max_pages, int page_rows, int64_t n_pages, int max_rank, void *workspace,
+                    int64_t workspace_bytes, void *stream)
+{
+    return sgmv_common(nullptr, nullptr, nullptr, nullptr, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank,
+                       scaling, T, 8, 8, n_adapters, max_pages, page_rows, n_pages, max_rank, MLORA_F16, 0, workspace,
+                       workspace_bytes, mlora::SGMV_PLAN, stream);
+}
+
+int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
+                       const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
+                       const int32_t *rank, const float *scaling, int T, int hin, int hout,
+                       int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                       int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return sgmv_common(y, x, a_rows, b_rows, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T, hin,
+                       hout, n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
+                       workspace_bytes, mlora::SGMV_APPLY, stream);
 }
 
 int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void *B_T, int B, int Lpad, int L,
@@ -317,7 +356,7 @@ int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void 
     a.b_rows = static_cast<const uint16_t *>(B_T) + (size_t)layer_idx * hout * r;
     a.n_seg = B; a.T = T; a.hin = hin; a.hout = hout; a.accumulate = 0; a.b_transposed = 1; a.seg_uniform_len = Lpad;
     carve(a, workspace, w);
-    rc = mlora::launch_sgmv(a, dtype, r, static_cast<hipStream_t>(stream));
+    rc = mlora::launch_sgmv(a, dtype, r, mlora::SGMV_PLAN | mlora::SGMV_APPLY, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "prefill launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
 }

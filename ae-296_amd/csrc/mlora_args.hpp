@@ -12,6 +12,10 @@ constexpr int MAX_RANK = 64;
 // [2] rank, [3] scaling (float bits), [4..11] token ids, [12..15] zero, [16..79] row of rank row j (-1 = absent).
 constexpr int WORK_WORDS = 80;
 constexpr int WORK_ROWS_AT = 16;
+// Prefill tile record (int32 words): [0] tokens in the tile (0 = nothing to do), [1] adapter (-1 = none),
+// [2] rank, [3] scaling (float bits), [4] first token, [5] segment, [6..15] zero, [16..79] row of rank row j.
+constexpr int TILE_WORDS = 80;
+constexpr int TILE_ROWS_AT = 16;
 
 // How the rank rows of an adapter are found inside a rows slab.
 struct PoolView {
@@ -83,6 +87,7 @@ struct SgmvArgs {
     int32_t *tile_tok0;
     int32_t *tile_ntok;
     int32_t *n_tiles;      // [1]
+    int32_t *tile_rec;     // [max_tiles * TILE_WORDS] per-tile records (layout below)
     float *v;              // [ksplit, T, MAX_RANK] fp32 partial intermediates
     uint16_t *vhi;         // [T, MAX_RANK] 16-bit hi part of the summed intermediate
     uint16_t *vlo;         // [T, MAX_RANK] 16-bit lo part
@@ -93,6 +98,8 @@ struct SgmvArgs {
 // launchers (defined next to their kernels); return hipError_t as int
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
 int launch_gather(const GatherArgs &a, hipStream_t s);
-int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, hipStream_t s);
+constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
+constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)
+int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s);
 
 }  // namespace mlora

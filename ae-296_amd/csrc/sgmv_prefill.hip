@@ -1,15 +1,16 @@
 // SGMV prefill kernels for gfx950: tokens are packed per segment (one adapter per segment)
 //     y[t] (+)= s_a * (x[t] . A_a) . B_a
-// computed on v_mfma_f32_16x16x32_{f16,bf16} tiles in four launches on one stream:
+// computed on v_mfma_f32_16x16x32_{f16,bf16} tiles in four launches on one stream (the first can be shared by all projections and layers of a batch):
 //   plan   : cuts every segment into tiles of 64 tokens (work list in the workspace);
 //   shrink : V[split][t][0..R) = x[t, Kslice] . A_a[:, Kslice]^T   (split-K, fp32 partials);
 //   reduce : sums the K splits and stores the result as a hi + lo pair of 16-bit values, so
 //            the intermediate keeps fp32 accuracy through the second MFMA;
 //   expand : y[t, cols] (+)= s_a * (Vhi + Vlo) . B_a[:, cols].
 // Both MFMA operands of the shrink are read straight from global memory in operand layout
-// (8 contiguous K values per lane).  The expand stages the B tile through LDS (rank must
-// be the in-lane K dimension, the pool stores rank rows) and writes y through a wave-private
-// LDS transpose so that every y access is a 16-byte, row-contiguous one.
+// (8 contiguous K values per lane).  The expand parks the B tile in LDS (rank must be the
+// in-lane K dimension, the pool stores rank rows), reads it back with the transposing LDS read,
+// and passes the output through a wavefront-private LDS tile so that every y access is a
+// 16-byte, row-contiguous one (8-byte accesses straight from the accumulators were measured slower).
 //
 // Replaces torch.bmm(torch.bmm(x, A), B) at lightllm/models/lora_gpu.py:127-128,145-146,157-158.
 #include "mlora_args.hpp"
@@ -21,6 +22,8 @@ constexpr int TM = 64;       // tokens per tile
 constexpr int TN = 128;      // output columns per expand step
 constexpr int SG_NT = 256;   // 4 wavefronts, 16 tokens each
 constexpr int VSTRIDE = MAX_RANK;
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4_t lds_short4;
 
 __device__ __forceinline__ int sg_pool_row(const int32_t *__restrict__ tbl, long long dense_stride, int adapter, int j,
                                            const PoolView &pv, long long n_rows)
@@ -78,7 +81,45 @@ __global__ __launch_bounds__(1024) void sgmv_plan_kernel(const SgmvArgs p)
         if (tid == 1023) s_carry = base + v;
         __syncthreads();
     }
-    if (tid == 0) p.n_tiles[0] = s_carry < p.max_tiles ? s_carry : p.max_tiles;
+    const int n_tiles = s_carry < p.max_tiles ? s_carry : p.max_tiles;
+    if (tid == 0) p.n_tiles[0] = n_tiles;
+    __syncthreads();                               // tile_* written above are visible to the whole block
+    // Per-tile records: everything a shrink / expand workgroup needs, so that it starts from one load.
+    // Headers of up to 1024 tiles at a time go through LDS (one tile per thread), then all threads
+    // fill the 80-word records of that batch with one table lookup per row word.
+    const PoolView &pv = p.pool;
+    __shared__ int s_hdr[1024][6];
+    for (int t0 = 0; t0 < n_tiles; t0 += 1024) {
+        const int t = t0 + tid;
+        if (t < n_tiles) {
+            const int seg = p.tile_seg[t];
+            int sstart, slen, adapter;
+            seg_of(p, seg, sstart, slen, adapter);
+            const bool real = adapter >= 0 && adapter < pv.n_adapters;
+            int rk = 0, sc = 0;
+            if (real) {
+                rk = pv.rank ? pv.rank[adapter] : pv.uniform_rank;
+                rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk);
+                if (pv.a_tbl) { const int cap = pv.max_pages << pv.page_shift; rk = rk > cap ? cap : rk; }
+                sc = __builtin_bit_cast(int, pv.scaling ? pv.scaling[adapter] : pv.uniform_scale);
+            }
+            s_hdr[tid][0] = p.tile_ntok[t]; s_hdr[tid][1] = real ? adapter : -1; s_hdr[tid][2] = rk;
+            s_hdr[tid][3] = sc; s_hdr[tid][4] = p.tile_tok0[t]; s_hdr[tid][5] = seg;
+        }
+        __syncthreads();
+        const int nb = n_tiles - t0 < 1024 ? n_tiles - t0 : 1024;
+        for (int idx = tid; idx < nb * TILE_WORDS; idx += 1024) {
+            const int lt = idx / TILE_WORDS, w = idx - lt * TILE_WORDS;
+            int val = 0;
+            if (w < 6) val = s_hdr[lt][w];
+            else if (w >= TILE_ROWS_AT) {
+                const int j = w - TILE_ROWS_AT, adapter = s_hdr[lt][1];
+                val = (adapter >= 0 && j < s_hdr[lt][2]) ? sg_pool_row(pv.a_tbl, pv.a_dense_stride, adapter, j, pv, pv.n_rows_a) : -1;
+            }
+            p.tile_rec[(size_t)(t0 + lt) * TILE_WORDS + w] = val;
+        }
+        __syncthreads();
+    }
 }
 
 // ------------------------------------------------------------------ shrink
@@ -94,76 +135,94 @@ __device__ __forceinline__ float4_t mfma16(const uint4 &a, const uint4 &b, float
 template <int DT, int RMAX>
 __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
 {
-    constexpr int NB = RMAX / 16;   // rank blocks of 16
-    constexpr int KU = 4;           // K steps (of 32) in flight
-    __shared__ int s_arow[RMAX];
+    // One workgroup: 64 tokens x RMAX ranks over one K slice.  A stage is 128 columns: the X tile
+    // (64 rows x 256 B) and the A tile (RMAX rows x 256 B) are read with 16-byte loads in which every
+    // 16-lane row covers 256 contiguous bytes, parked in LDS, and consumed from there as MFMA operands
+    // (8 contiguous K values per lane).  The next stage's loads are in flight while this one computes.
+    constexpr int NB = RMAX / 16;            // rank blocks of 16
+    constexpr int KB = 128;                  // columns per stage
+    constexpr int CPR = KB / 8;              // 16-byte chunks per row and stage
+    constexpr int PITCH = KB * 2 + 16;       // LDS row pitch in bytes (keeps operand reads spread over the banks)
+    constexpr int XP = TM * CPR / SG_NT;     // X loads per thread and stage (4)
+    constexpr int AP = (RMAX * CPR + SG_NT - 1) / SG_NT;   // A loads per thread and stage (1, 2 or 4)
+    __shared__ __attribute__((aligned(16))) unsigned char s_x[TM * PITCH];
+    __shared__ __attribute__((aligned(16))) unsigned char s_a[RMAX * PITCH];
     const int tile = blockIdx.x, split = blockIdx.y;
     if (tile >= p.n_tiles[0]) return;
-    const int seg = p.tile_seg[tile];
-    int sstart, slen, adapter;
-    seg_of(p, seg, sstart, slen, adapter);
-    const PoolView &pv = p.pool;
-    if (adapter < 0 || adapter >= pv.n_adapters) return;
-    const int tok0 = p.tile_tok0[tile], ntok = p.tile_ntok[tile];
-    if (ntok <= 0 || tok0 < 0 || tok0 + ntok > p.T) return;
-    int r = pv.rank ? pv.rank[adapter] : pv.uniform_rank;
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    if (pv.a_tbl) { const int cap = pv.max_pages << pv.page_shift; r = r > cap ? cap : r; }
+    const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
+    const int ntok = rec[0], adapter = rec[1];
+    const int tok0 = rec[4];
+    if (adapter < 0 || ntok <= 0 || tok0 < 0 || tok0 + ntok > p.T) return;
+    const int32_t *__restrict__ rows = rec + TILE_ROWS_AT;     // -1 for every rank row that does not exist
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 15, g = lane >> 4;
-    for (int j = tid; j < RMAX; j += SG_NT)
-        s_arow[j] = j < r ? sg_pool_row(pv.a_tbl, pv.a_dense_stride, adapter, j, pv, pv.n_rows_a) : -1;
-    __syncthreads();
 
     const int hin = p.hin;
     const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x);
     const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows);
-    int trow = wave * 16 + m;
-    trow = trow < ntok ? trow : ntok - 1;                       // tail rows recompute the last token; never stored
-    const uint4 *xp = reinterpret_cast<const uint4 *>(x + (size_t)(tok0 + trow) * hin);
-    const uint4 *ap[NB];
+    const int lrow = tid >> 4, lchk = tid & 15;                // this thread's row (per pass of 16) and chunk
+    const uint4 *xp[XP];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        const int row = s_arow[nb * 16 + m];
-        ap[nb] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+    for (int q = 0; q < XP; q++) {
+        int t = lrow + 16 * q;
+        t = t < ntok ? t : ntok - 1;                            // tail rows repeat the last token; never stored
+        xp[q] = reinterpret_cast<const uint4 *>(x + (size_t)(tok0 + t) * hin);
+    }
+    const uint4 *ap[AP];
+#pragma unroll
+    for (int q = 0; q < AP; q++) {
+        const int j = lrow + 16 * q;
+        const int row = j < RMAX ? rows[j] : -1;
+        ap[q] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
     }
     float4_t acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int ncc = hin >> 3;                                   // 16-byte chunks per row
-    const int ksteps = (ncc + 3) >> 2;
-    const int per = (ksteps + p.ksplit - 1) / p.ksplit;
-    const int ks0 = split * per;
-    const int ks1 = ks0 + per < ksteps ? ks0 + per : ksteps;
-#pragma unroll 1
-    for (int ks = ks0; ks < ks1; ks += KU) {
-        uint4 xf[KU], af[KU][NB];
+    const int nstage = (ncc + CPR - 1) / CPR;
+    const int per = (nstage + p.ksplit - 1) / p.ksplit;
+    const int st0 = split * per;
+    const int st1 = st0 + per < nstage ? st0 + per : nstage;
+    uint4 xr[XP], ar[AP];
+    auto load_stage = [&](int st) {
+        const int c = st * CPR + lchk;
+        const bool ok = c < ncc;                                // K tail: both operands become zero
+        const int cs = ok ? c : ncc - 1;
 #pragma unroll
-        for (int u = 0; u < KU; u++) {
-            const int c = (ks + u) * 4 + g;
-            const bool ok = (ks + u) < ks1 && c < ncc;
-            const int cs = c < ncc ? c : ncc - 1;
-            xf[u] = xp[cs];
-            if (!ok) xf[u] = zero16();
+        for (int q = 0; q < XP; q++) { xr[q] = xp[q][cs]; if (!ok) xr[q] = zero16(); }
+#pragma unroll
+        for (int q = 0; q < AP; q++) { ar[q] = ap[q][cs]; if (!ok) ar[q] = zero16(); }
+    };
+    if (st0 < st1) load_stage(st0);
+#pragma unroll 1
+    for (int st = st0; st < st1; st++) {
+        __syncthreads();                                        // the previous stage has been consumed
+#pragma unroll
+        for (int q = 0; q < XP; q++)
+            *reinterpret_cast<uint4 *>(s_x + (lrow + 16 * q) * PITCH + lchk * 16) = xr[q];
+#pragma unroll
+        for (int q = 0; q < AP; q++)
+            if (lrow + 16 * q < RMAX) *reinterpret_cast<uint4 *>(s_a + (lrow + 16 * q) * PITCH + lchk * 16) = ar[q];
+        __syncthreads();
+        if (st + 1 < st1) load_stage(st + 1);
+#pragma unroll
+        for (int ks = 0; ks < KB / 32; ks++) {
+            const uint4 xf = *reinterpret_cast<const uint4 *>(s_x + (wave * 16 + m) * PITCH + (ks * 4 + g) * 16);
 #pragma unroll
             for (int nb = 0; nb < NB; nb++) {
-                af[u][nb] = ap[nb][cs];
-                if (!ok) af[u][nb] = zero16();
+                const uint4 af = *reinterpret_cast<const uint4 *>(s_a + (nb * 16 + m) * PITCH + (ks * 4 + g) * 16);
+                acc[nb] = mfma16<DT>(xf, af, acc[nb]);
             }
         }
-#pragma unroll
-        for (int u = 0; u < KU; u++)
-#pragma unroll
-            for (int nb = 0; nb < NB; nb++) acc[nb] = mfma16<DT>(xf[u], af[u][nb], acc[nb]);
     }
     // D[token 4g+i][rank m] per 16x16 block; rank columns that do not exist are stored as zero.
     float *vout = p.v + ((size_t)split * p.T + tok0 + wave * 16) * VSTRIDE;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
         const int col = nb * 16 + m;
-        const bool col_ok = s_arow[col] >= 0;
+        const bool col_ok = rows[col] >= 0;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int trow_o = wave * 16 + 4 * g + i;
@@ -216,22 +275,31 @@ __global__ __launch_bounds__(256) void sgmv_reduce_kernel(const SgmvArgs p)
 template <int DT, int RMAX, bool BT>
 __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, int cols_per_block)
 {
+    // One workgroup: 64 tokens (16 per wavefront) x cols_per_block output columns, 128 columns per step.
+    // The B tile of a step is parked in LDS row-major and read back column-wise with the transposing LDS
+    // read (the MFMA needs rank as the in-lane K dimension, the pool stores rank rows).  The 16 x 128
+    // result of a wavefront goes through a wavefront-private LDS tile so that y is read and written with
+    // 16-byte accesses in which a 16-lane row covers 256 contiguous bytes of one token.  Loads of y and B
+    // run one step ahead of the arithmetic.
     constexpr int KP = RMAX <= 32 ? 32 : 64;   // K of the expand MFMAs (rank padded with zeros)
     constexpr int KS = KP / 32;
     constexpr int NBC = TN / 16;               // 16-column blocks per step
-    constexpr int BPITCH = TN * 2 + 4;         // bytes per rank row of the LDS B tile
+    constexpr int BPITCH = TN * 2 + 16;        // bytes per rank row of the LDS B tile (16-byte aligned rows)
     constexpr int OPITCH = TN + 4;             // floats per token row of the staging tile
+    constexpr int BQ = BT ? 1 : KP * (TN / 8) / SG_NT;   // B-tile loads per thread and step
     __shared__ __attribute__((aligned(16))) unsigned char s_b[BT ? 16 : KP * BPITCH];
     __shared__ __attribute__((aligned(16))) float s_out[SG_NT / 64][16][OPITCH];
     __shared__ int s_brow[BT ? 1 : KP];
+    typedef __attribute__((address_space(3))) volatile float lds_vfloat;
+    typedef __attribute__((address_space(3))) volatile float4_t lds_vfloat4;
 
     const int tile = blockIdx.x;
     if (tile >= p.n_tiles[0]) return;
-    const int seg = p.tile_seg[tile];
-    int sstart, slen, adapter;
-    seg_of(p, seg, sstart, slen, adapter);
+    const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
+    const int ntok = rec[0], adapter = rec[1], r = rec[2];
+    const float scale = __builtin_bit_cast(float, rec[3]);
+    const int tok0 = rec[4];
     const PoolView &pv = p.pool;
-    const int tok0 = p.tile_tok0[tile], ntok = p.tile_ntok[tile];
     if (ntok <= 0 || tok0 < 0 || tok0 + ntok > p.T) return;
     const int hout = p.hout;
     uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y);
@@ -241,7 +309,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     int col_end = col_begin + cols_per_block;
     col_end = col_end < hout ? col_end : hout;
 
-    if (adapter < 0 || adapter >= pv.n_adapters) {
+    if (adapter < 0) {
         if (!p.accumulate) {
             // segment without adapter: y = delta means zeros
             const int cpr = (col_end - col_begin) >> 3;
@@ -252,14 +320,12 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
         }
         return;
     }
-    int r = pv.rank ? pv.rank[adapter] : pv.uniform_rank;
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    if (pv.a_tbl) { const int cap = pv.max_pages << pv.page_shift; r = r > cap ? cap : r; }
-    const float scale = pv.scaling ? pv.scaling[adapter] : pv.uniform_scale;
-
     if constexpr (!BT) {
-        for (int j = tid; j < KP; j += SG_NT)
-            s_brow[j] = j < r ? sg_pool_row(pv.b_tbl, pv.b_dense_stride, adapter, j, pv, pv.n_rows_b) : -1;
+        // B rows share the page table with the A rows
+        for (int j = tid; j < KP; j += SG_NT) {
+            const int row = j < MAX_RANK ? rec[TILE_ROWS_AT + j] : -1;
+            s_brow[j] = (row >= 0 && row < pv.n_rows_b) ? row : -1;
+        }
     }
 
     // ---- V operand: 16 tokens of this wavefront x KP ranks as a hi + lo pair of 16-bit values
@@ -280,33 +346,48 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     const uint16_t *__restrict__ bt = brows + (BT ? (size_t)adapter * (size_t)pv.b_dense_stride : 0);
     __syncthreads();
 
-#pragma unroll 1
-    for (int col0 = col_begin; col0 < col_end; col0 += TN) {
-        // y rows of this wavefront: lane handles (token p / 16, 16-byte chunk p % 16), p = lane + 64 q
-        uint4 y0[4];
+    // Loads of a step (this thread's share of the B tile and of the y rows) are issued one step ahead.
+    // y rows of this wavefront: lane handles (token p / 16, 16-byte chunk p % 16), p = lane + 64 q.
+    uint4 y_nx[4], b_nx[BQ];
+    auto prefetch = [&](int col0) {
         if (p.accumulate) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int pp = lane + 64 * q, t = pp >> 4, c = pp & 15;
                 const int col = col0 + c * 8;
                 const bool ok = wave * 16 + t < ntok && col < col_end;
-                y0[q] = ok ? ldg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col) : zero16();
+                y_nx[q] = ok ? ldg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col) : zero16();
             }
         }
         if constexpr (!BT) {
-            // stage B[0..KP) x [col0, col0+TN) in LDS, rows beyond the rank as zeros
-            __syncthreads();
-            for (int e = tid; e < KP * (TN / 8); e += SG_NT) {
+#pragma unroll
+            for (int q = 0; q < BQ; q++) {
+                const int e = tid + q * SG_NT;
                 const int j = e / (TN / 8), c = e - j * (TN / 8);
                 const int row = s_brow[j];
                 const int col = col0 + c * 8;
-                uint4 bv = zero16();
-                if (row >= 0 && col < col_end) bv = ldg16(brows + (size_t)row * hout + col);
-                uint32_t *dst = reinterpret_cast<uint32_t *>(s_b + j * BPITCH + c * 16);
-                dst[0] = bv.x; dst[1] = bv.y; dst[2] = bv.z; dst[3] = bv.w;
+                b_nx[q] = (row >= 0 && col < col_end) ? ldg16(brows + (size_t)row * hout + col) : zero16();
+            }
+        }
+    };
+    prefetch(col_begin);
+#pragma unroll 1
+    for (int col0 = col_begin; col0 < col_end; col0 += TN) {
+        uint4 y0[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) y0[q] = y_nx[q];
+        if constexpr (!BT) {
+            // park B[0..KP) x [col0, col0+TN) in LDS, rows beyond the rank as zeros
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < BQ; q++) {
+                const int e = tid + q * SG_NT;
+                const int j = e / (TN / 8), c = e - j * (TN / 8);
+                *reinterpret_cast<uint4 *>(s_b + j * BPITCH + c * 16) = b_nx[q];
             }
             __syncthreads();
         }
+        if (col0 + TN < col_end) prefetch(col0 + TN);
         float4_t acc[NBC];
 #pragma unroll
         for (int nb = 0; nb < NBC; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -316,42 +397,43 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
             for (int ks = 0; ks < KS; ks++) {
                 uint4 bop;
                 if constexpr (!BT) {
-                    // lane (n = m, k group g): B[ks*32 + 8g + e][col0 + nb*16 + m], e < 8
-                    const unsigned char *src = s_b + (ks * 32 + 8 * g) * BPITCH + (nb * 16 + m) * 2;
-                    uint32_t h[8];
-#pragma unroll
-                    for (int e = 0; e < 8; e++) h[e] = *reinterpret_cast<const uint16_t *>(src + e * BPITCH);
-                    bop = make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16));
+                    // lane (n = m, k group g) needs B[ks*32 + 8g + e][nb*16 + m], e < 8: a column of the row-major
+                    // tile.  ds_read_b64_tr_b16 does the transpose: the 16 lanes of a group read a 4 x 16 block
+                    // (lane i: row i / 4, columns 4 (i % 4) ..+3) and lane n gets the 4 rows of column n.
+                    const unsigned char *src = s_b + (ks * 32 + 8 * g + (m >> 2)) * BPITCH + (nb * 16 + (m & 3) * 4) * 2;
+                    const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4 *)src);
+                    const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4 *)(src + 4 * BPITCH));
+                    bop = make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
+                                     __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
                 } else {
                     const int col = col0 + nb * 16 + m;
                     const int k0 = ks * 32 + 8 * g;
                     bop = (col < col_end && k0 < r) ? ldg16(bt + (size_t)col * r + k0) : zero16();
                 }
-                // D[m = column][n = token] would scatter y; keep D[token][column]: A operand = V, B operand = B
+                // D[token 4g+i][column m of the block]: A operand = V, B operand = B
                 acc[nb] = mfma16<DT>(vhi[ks], bop, acc[nb]);
                 acc[nb] = mfma16<DT>(vlo[ks], bop, acc[nb]);
             }
         }
-        // ---- transpose through LDS (one 16 x TN tile per wavefront), then 16-byte row-contiguous y update
+        // ---- transpose through this wavefront's own LDS tile, then 16-byte row-contiguous y update.
+        // The tile is private to the wavefront and LDS operations of one wavefront complete in order, so no
+        // barrier is needed; the accesses are volatile so that the compiler keeps them in program order and
+        // emits one ds_write_b32 per element (left to itself it pairs these stores into ds_write2_b32 and,
+        // in the variant without the B tile, gets two of the paired offsets wrong).
         {
-            // volatile: one ds_write_b32 per element.  Left to itself the compiler pairs these
-            // stores into ds_write2_b32 and, in the variant without the B staging tile, gets two
-            // of the paired offsets wrong.
-            typedef __attribute__((address_space(3))) volatile float lds_vfloat;
             lds_vfloat *so = (lds_vfloat *)&s_out[wave][4 * g][m];
 #pragma unroll
             for (int nb = 0; nb < NBC; nb++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) so[i * OPITCH + nb * 16] = acc[nb][i];
         }
-        __syncthreads();
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int pp = lane + 64 * q, t = pp >> 4, c = pp & 15;
             const int col = col0 + c * 8;
+            const float4_t d0 = *(lds_vfloat4 *)&s_out[wave][t][c * 8];
+            const float4_t d1 = *(lds_vfloat4 *)&s_out[wave][t][c * 8 + 4];
             if (wave * 16 + t < ntok && col < col_end) {
-                const float4_t d0 = *reinterpret_cast<const float4_t *>(&s_out[wave][t][c * 8]);
-                const float4_t d1 = *reinterpret_cast<const float4_t *>(&s_out[wave][t][c * 8 + 4]);
                 float o[8];
                 if (p.accumulate) unpack8<DT>(y0[q], o);
                 else {
@@ -365,16 +447,19 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
                 stg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col, pack8<DT>(o));
             }
         }
-        if constexpr (BT) __syncthreads();   // staging tile is rewritten by the next step (the B staging barrier covers !BT)
     }
 }
 
 template <int DT, int RMAX>
-static int launch_rmax(const SgmvArgs &a, hipStream_t s)
+static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
 {
-    hipLaunchKernelGGL(sgmv_plan_kernel, dim3(1), dim3(1024), 0, s, a);
-    int rc = (int)hipGetLastError();
-    if (rc) return rc;
+    int rc = 0;
+    if (phases & SGMV_PLAN) {
+        hipLaunchKernelGGL(sgmv_plan_kernel, dim3(1), dim3(1024), 0, s, a);
+        rc = (int)hipGetLastError();
+        if (rc) return rc;
+    }
+    if (!(phases & SGMV_APPLY)) return 0;
     hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3(a.max_tiles, a.ksplit), dim3(SG_NT), 0, s, a);
     rc = (int)hipGetLastError();
     if (rc) return rc;
@@ -396,17 +481,17 @@ static int launch_rmax(const SgmvArgs &a, hipStream_t s)
 }
 
 template <int DT>
-static int launch_sg_dt(const SgmvArgs &a, int max_rank, hipStream_t s)
+static int launch_sg_dt(const SgmvArgs &a, int max_rank, int phases, hipStream_t s)
 {
-    if (max_rank <= 16) return launch_rmax<DT, 16>(a, s);
-    if (max_rank <= 32) return launch_rmax<DT, 32>(a, s);
-    return launch_rmax<DT, 64>(a, s);
+    if (max_rank <= 16) return launch_rmax<DT, 16>(a, phases, s);
+    if (max_rank <= 32) return launch_rmax<DT, 32>(a, phases, s);
+    return launch_rmax<DT, 64>(a, phases, s);
 }
 
-int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, hipStream_t s)
+int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s)
 {
-    if (dtype == DT_F16) return launch_sg_dt<DT_F16>(a, max_rank, s);
-    return launch_sg_dt<DT_BF16>(a, max_rank, s);
+    if (dtype == DT_F16) return launch_sg_dt<DT_F16>(a, max_rank, phases, s);
+    return launch_sg_dt<DT_BF16>(a, max_rank, phases, s);
 }
 
 }  // namespace mlora

@@ -7,9 +7,9 @@ and raises if it has not been built.
 from . import _ext
 from ._ext import MloraError
 from .lora_gpu import Lora_GPU
-from .ops import (DecodePlan, add_lora_bgmv, bgmv, lora_apply, lora_prefill_ref, plan_decode, sgmv,
-                  sgmv_workspace)
+from .ops import (DecodePlan, PrefillPlan, add_lora_bgmv, bgmv, lora_apply, lora_prefill_ref, plan_decode,
+                  plan_prefill, sgmv, sgmv_workspace)
 from .pool import AdapterPool
 
 __all__ = ["AdapterPool", "DecodePlan", "Lora_GPU", "MloraError", "add_lora_bgmv", "bgmv", "lora_apply",
-           "lora_prefill_ref", "plan_decode", "sgmv", "sgmv_workspace", "_ext"]
+           "lora_prefill_ref", "plan_decode", "plan_prefill", "PrefillPlan", "sgmv", "sgmv_workspace", "_ext"]

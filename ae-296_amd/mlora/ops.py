@@ -171,29 +171,68 @@ def sgmv_workspace(T: int, n_seg: int, device) -> torch.Tensor:
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
-def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: str,
-         seg_start: torch.Tensor, seg_len: torch.Tensor, seg_adapter: torch.Tensor,
-         accumulate: bool = True, workspace: Optional[torch.Tensor] = None) -> None:
-    """Prefill LoRA apply over packed segments (one adapter per segment) on MFMA tiles."""
-    _need_cuda(y, x, seg_start, seg_len, seg_adapter)
-    _need_contig(y, x, seg_start, seg_len, seg_adapter)
+@dataclass
+class PrefillPlan:
+    """Tile list and per-tile records of one prefill batch, held in `workspace` (written by ``mlora_sgmv_plan``)."""
+    seg_start: torch.Tensor
+    seg_len: torch.Tensor
+    seg_adapter: torch.Tensor
+    T: int
+    workspace: torch.Tensor
+
+
+def _check_segments(seg_start, seg_len, seg_adapter):
+    _need_cuda(seg_start, seg_len, seg_adapter)
+    _need_contig(seg_start, seg_len, seg_adapter)
     for s in (seg_start, seg_len, seg_adapter):
         if s.dtype != torch.int32:
             raise TypeError("segment arrays must be int32")
+    n_seg = seg_start.numel()
+    if seg_len.numel() != n_seg or seg_adapter.numel() != n_seg:
+        raise ValueError("seg_start, seg_len and seg_adapter must have the same length")
+    return n_seg
+
+
+def plan_prefill(seg_start: torch.Tensor, seg_len: torch.Tensor, seg_adapter: torch.Tensor, T: int,
+                 pool: AdapterPool, workspace: Optional[torch.Tensor] = None) -> PrefillPlan:
+    """Plan a prefill batch once; the plan serves every projection and layer (``sgmv(..., plan=plan)``)."""
+    n_seg = _check_segments(seg_start, seg_len, seg_adapter)
+    if workspace is None:
+        workspace = sgmv_workspace(T, n_seg, seg_start.device)
+    pool.sync()
+    rc = _ext.lib().mlora_sgmv_plan(
+        seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(), n_seg,
+        _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling), T, pool.n_slots, pool.max_pages,
+        pool.page_rows, pool.n_pages, pool.max_rank, workspace.data_ptr(), workspace.numel(), _ext.current_stream_ptr())
+    _ext.check(rc)
+    return PrefillPlan(seg_start, seg_len, seg_adapter, T, workspace)
+
+
+def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: str,
+         seg_start: Optional[torch.Tensor] = None, seg_len: Optional[torch.Tensor] = None,
+         seg_adapter: Optional[torch.Tensor] = None, accumulate: bool = True,
+         workspace: Optional[torch.Tensor] = None, plan: Optional[PrefillPlan] = None) -> None:
+    """Prefill LoRA apply over packed segments (one adapter per segment) on MFMA tiles.  Either pass the
+    segment arrays (planned inside the call) or a `plan` from ``plan_prefill``."""
+    if plan is not None:
+        seg_start, seg_len, seg_adapter, workspace = plan.seg_start, plan.seg_len, plan.seg_adapter, plan.workspace
+    _need_cuda(y, x)
+    _need_contig(y, x)
+    n_seg = _check_segments(seg_start, seg_len, seg_adapter)
     hin, hout = pool.projections[proj]
     T = x.shape[0]
+    if plan is not None and plan.T != T:
+        raise ValueError("plan was made for a different number of tokens")
     if tuple(x.shape) != (T, hin) or tuple(y.shape) != (T, hout):
         raise ValueError(f"expected x [{T}, {hin}] and y [{T}, {hout}]")
     if x.dtype != pool.dtype or y.dtype != pool.dtype:
         raise TypeError(f"x and y must have the pool dtype {pool.dtype}")
-    n_seg = seg_start.numel()
-    if seg_len.numel() != n_seg or seg_adapter.numel() != n_seg:
-        raise ValueError("seg_start, seg_len and seg_adapter must have the same length")
     if workspace is None:
         workspace = sgmv_workspace(T, n_seg, x.device)
     pool.sync()
     a_ptr, b_ptr = pool.slab_ptrs(layer, proj)
-    rc = _ext.lib().mlora_sgmv(
+    fn = _ext.lib().mlora_sgmv_planned if plan is not None else _ext.lib().mlora_sgmv
+    rc = fn(
         y.data_ptr(), x.data_ptr(), a_ptr, b_ptr, seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(),
         n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
         T, hin, hout, pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.max_rank,

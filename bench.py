@@ -89,8 +89,9 @@ def bench_c4(args, dev):
     ws = mlora.sgmv_workspace(T, 16, dev)
 
     def step():
+        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)      # once per batch, shared by the projections
         for p, (hin, hout) in projections.items():
-            mlora.sgmv(y[p], x[hin], pool, 0, p, ss, sl, sa, accumulate=True, workspace=ws)
+            mlora.sgmv(y[p], x[hin], pool, 0, p, accumulate=True, plan=plan)
 
     step()
     torch.cuda.synchronize()

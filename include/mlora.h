@@ -170,6 +170,25 @@ int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
                int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * The same in two parts, for the usual case in which one batch of segments is applied to many
+ * projections and layers: mlora_sgmv_plan writes the tile list and per-tile records (tokens, adapter,
+ * rank, scaling, row of every rank row) into the workspace once; mlora_sgmv_planned then runs the
+ * arithmetic of one projection against that plan.  The segments, pool tables, T and workspace must be
+ * the ones the plan was made with; the plan stays valid until the page table, rank or scaling of a
+ * planned adapter changes.  No counterpart in the reference (its prefill re-derives everything per call).
+ */
+int mlora_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                    const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                    int T, int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                    void *workspace, int64_t workspace_bytes, void *stream);
+int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b_rows,
+                       const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                       const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                       int T, int hin, int hout, int n_adapters, int max_pages, int page_rows,
+                       int64_t n_pages, int max_rank,
+                       int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * The reference's prefill call on its own layout (lora_gpu.py:125-128): request b uses
  * adapter slot b; x [B, Lpad, hin]; A_T [>=B, L, r, hin]; B_T [>=B, L, hout, r];
  * y [B, Lpad, hout] = (x[b] . A_T[b, layer]^T) . B_T[b, layer]^T   (y is overwritten).

@@ -6,7 +6,7 @@ import torch
 
 from gpu_common import ATOL, RTOL, assert_close_bits, oracle_apply, say, tdtype, upload_pool
 from helpers import BF16, FP16, PagedPool, bits_of, bits_to_torch, f32_of, torch_to_bits
-from mlora import bgmv, sgmv
+from mlora import bgmv, plan_prefill, sgmv
 
 pytestmark = pytest.mark.gpu
 
@@ -111,6 +111,36 @@ def test_sgmv_segments_without_adapter_and_gaps():
     assert np.all(got_d[10:40] == 0)                       # adapter-less segment is defined as zeros
     covered = tok >= 0
     assert_close_bits(got_d[covered], oracle_apply(pp, x, tok, None)[covered], FP16)
+
+
+def test_sgmv_plan_once_apply_many():
+    """One plan serves several projections and layers, and matches the self-planning call bit for bit."""
+    rng = np.random.default_rng(73)
+    ranks = [64, 16, 32, 8]
+    hin, hout = 512, 768
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=BF16)
+    from mlora import AdapterPool
+    pool = upload_pool(pp, projections={"p": (hin, hout), "o": (hout, hin)}, n_layers=2)
+    for l in range(2):
+        pool.a_rows["o"][l].normal_(0, 0.02)
+        pool.b_rows["o"][l].normal_(0, 0.02)
+    pool.a_rows["p"][1].normal_(0, 0.02)
+    pool.b_rows["p"][1].normal_(0, 0.02)
+    lens = [70, 3, 128, 65]
+    ss, sl, sa = (torch.from_numpy(a).cuda() for a in _segments(lens, [2, 0, 3, 1]))
+    T = sum(lens)
+    say("sgmv: one plan, two layers x two projections")
+    plan = plan_prefill(ss, sl, sa, T, pool)
+    for l in range(2):
+        for proj, (hi, ho) in (("p", (hin, hout)), ("o", (hout, hin))):
+            x = torch.randn(T, hi, device="cuda").bfloat16()
+            y0 = torch.randn(T, ho, device="cuda").bfloat16()
+            y_plan, y_self = y0.clone(), y0.clone()
+            sgmv(y_plan, x, pool, l, proj, plan=plan)
+            sgmv(y_self, x, pool, l, proj, ss, sl, sa)
+            torch.cuda.synchronize()
+            assert torch.equal(y_plan, y_self)
+            assert not torch.equal(y_plan, y0)
 
 
 def test_sgmv_equals_bgmv_at_config4_size():
