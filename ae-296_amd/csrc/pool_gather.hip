@@ -14,12 +14,11 @@
 
 namespace mlora {
 
-constexpr int GATHER_NT = 1024;
+constexpr int GATHER_NT_MAX = 1024;
 constexpr int GATHER_MAX_T = 8192;
 constexpr int TOK_BITS = 13;                 // token id field of the sort key
-constexpr int EPT = GATHER_MAX_T / GATHER_NT;  // sorted positions per thread in the scans
 
-// Inclusive scan over GATHER_NT per-thread values; op = 0 sum, 1 max, 2 min.
+// Inclusive scan over the block's per-thread values; op = 0 sum, 1 max, 2 min.
 template <int OP>
 __device__ __forceinline__ int scan_op(int a, int b)
 {
@@ -45,8 +44,13 @@ __device__ int block_scan_inclusive(int v, int identity, int *s_wave /* [16] */)
     return scan_op<OP>(base, v);
 }
 
+// One workgroup of GATHER_NT threads groups up to MAXT tokens (EPT sorted positions per thread in the
+// scans).  The MAXT = 2048 instance also keeps the chunk headers in LDS, which makes writing the work
+// records cheap; decode batches are normally that small.
+template <int GATHER_NT, int MAXT>
 __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
 {
+    constexpr int EPT = MAXT / GATHER_NT;
     const int tid = threadIdx.x;
     if (blockIdx.x > 0) {
         // ---- per-token view
@@ -75,7 +79,10 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
     if (!g.perm) return;
 
     // ---- grouped view (one workgroup)
-    __shared__ uint32_t s_key[GATHER_MAX_T];
+    constexpr bool LDS_HDR = MAXT <= 2048;                 // chunk headers fit in LDS next to the keys
+    __shared__ uint32_t s_key[MAXT];
+    __shared__ int s_chdr[LDS_HDR ? MAXT : 1];             // start | len << 13 | rank << 17 per chunk
+    __shared__ float s_cscale[LDS_HDR ? MAXT : 1];
     __shared__ int s_wave[16];
     __shared__ int s_cnt[2];
     const int T = g.T;
@@ -192,9 +199,19 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         }
         if (chead[e]) {
             const int left = segend[e] - i;
+            const int len = left < g.group ? left : g.group;
             g.chunk_start[ch_idx] = i;
-            g.chunk_len[ch_idx] = left < g.group ? left : g.group;
+            g.chunk_len[ch_idx] = len;
             g.chunk_adapter[ch_idx] = real ? ad[e] : -1;
+            if constexpr (LDS_HDR) {
+                if (g.work) {
+                    int rk = 0;
+                    float sc = 0.f;
+                    if (real) { rk = g.rank[ad[e]]; rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); sc = g.scaling[ad[e]]; }
+                    s_chdr[ch_idx] = i | (len << TOK_BITS) | (rk << (TOK_BITS + 4));
+                    s_cscale[ch_idx] = sc;
+                }
+            }
             ch_idx++;
         }
     }
@@ -206,6 +223,47 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         __syncthreads();                         // chunk_* arrays written above are visible to the whole block
         const int n_chunks = s_nchunks;
         const int per_xcd = (n_chunks + 7) >> 3;
+        if constexpr (LDS_HDR) {
+            // 16 bytes per step: header quad, two token quads, a zero quad, then 16 quads of row indices.
+            constexpr int QPR = WORK_WORDS / 4;
+            int4 *out = reinterpret_cast<int4 *>(g.work);
+            const int quads = g.work_cap * QPR;
+            const uint32_t tmask = (1u << TOK_BITS) - 1u;
+#pragma unroll 4
+            for (int q = tid; q < quads; q += GATHER_NT) {
+                const int b = q / QPR, w4 = q - b * QPR;
+                const int c = (b & 7) * per_xcd + (b >> 3);
+                int4 v = make_int4(0, w4 == 0 ? -1 : 0, 0, 0);
+                if ((b >> 3) < per_xcd && c < n_chunks) {
+                    const int hdr = s_chdr[c];
+                    const int start = hdr & (int)tmask, len = (hdr >> TOK_BITS) & 15, rk = hdr >> (TOK_BITS + 4);
+                    int a = (int)(s_key[start] >> TOK_BITS);
+                    a = a < g.n_adapters ? a : -1;
+                    if (w4 == 0) v = make_int4(len, a, rk, __builtin_bit_cast(int, s_cscale[c]));
+                    else if (w4 <= 2) {
+                        const int k0 = (w4 - 1) * 4;
+                        v.x = k0 + 0 < len ? (int)(s_key[start + k0 + 0] & tmask) : -1;
+                        v.y = k0 + 1 < len ? (int)(s_key[start + k0 + 1] & tmask) : -1;
+                        v.z = k0 + 2 < len ? (int)(s_key[start + k0 + 2] & tmask) : -1;
+                        v.w = k0 + 3 < len ? (int)(s_key[start + k0 + 3] & tmask) : -1;
+                    } else if (w4 >= WORK_ROWS_AT / 4) {
+                        const int j0 = (w4 - WORK_ROWS_AT / 4) * 4;
+                        int rr[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int j = j0 + e;
+                            rr[e] = -1;
+                            if (a >= 0 && j < rk && j / g.page_rows < g.max_pages) {
+                                const int pg = g.page_tbl[(long long)a * g.max_pages + j / g.page_rows];
+                                if (pg >= 0 && pg < g.n_pages) rr[e] = pg * g.page_rows + j % g.page_rows;
+                            }
+                        }
+                        v = make_int4(rr[0], rr[1], rr[2], rr[3]);
+                    }
+                }
+                out[q] = v;
+            }
+        } else {
         const long long words = (long long)g.work_cap * WORK_WORDS;
         for (long long idx = tid; idx < words; idx += GATHER_NT) {
             const int b = (int)(idx / WORK_WORDS), w = (int)(idx - (long long)b * WORK_WORDS);
@@ -232,6 +290,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
             }
             g.work[idx] = val;
         }
+        }
     }
     if (tid == GATHER_NT - 1) {
         g.counters[0] = seg_incl;
@@ -245,8 +304,9 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
 int launch_gather(const GatherArgs &a, hipStream_t s)
 {
     const long long per_tok = (a.out_row_off || a.out_rank || a.out_scale) ? (long long)a.T * a.max_pages : 0;
-    const unsigned grid = 1u + (unsigned)((per_tok + GATHER_NT - 1) / GATHER_NT);
-    hipLaunchKernelGGL(gather_kernel, dim3(grid), dim3(GATHER_NT), 0, s, a);
+    const unsigned grid = 1u + (unsigned)((per_tok + GATHER_NT_MAX - 1) / GATHER_NT_MAX);
+    if (a.T <= 2048) hipLaunchKernelGGL((gather_kernel<GATHER_NT_MAX, 2048>), dim3(grid), dim3(GATHER_NT_MAX), 0, s, a);
+    else hipLaunchKernelGGL((gather_kernel<GATHER_NT_MAX, GATHER_MAX_T>), dim3(grid), dim3(GATHER_NT_MAX), 0, s, a);
     return (int)hipGetLastError();
 }
 

@@ -46,6 +46,28 @@ __device__ __forceinline__ void seg_of(const SgmvArgs &p, int s, int &start, int
     if (len > p.T - start) len = p.T - start;
 }
 
+// Workgroup id -> (tile, second index) for the shrink (second = K split) and the expand (second = column
+// block).  Workgroups are dealt to the 8 XCDs round-robin by id and every XCD has its own L2; tiles are
+// ordered by segment, so runs of XRUN consecutive tiles mostly share one adapter.  All workgroups of a
+// run that have the same second index read the same slice of A (or B): they are given ids with the same
+// residue mod 8, i.e. one XCD, and the residue rotates with the second index so the XCDs stay balanced.
+constexpr int XRUN = 8;
+__device__ __forceinline__ bool xcd_remap(int w, int n_second, int &tile, int &second)
+{
+    const int r = w & 7, slot = w >> 3;
+    const int i = slot % XRUN;
+    second = (slot / XRUN) % n_second;
+    const int j = slot / (XRUN * n_second);
+    const int run = ((r - second) & 7) + 8 * j;
+    tile = run * XRUN + i;
+    return true;
+}
+__host__ __device__ inline long long xcd_grid(int max_tiles, int n_second)
+{
+    const long long runs = (max_tiles + XRUN - 1) / XRUN;
+    return 8LL * ((runs + 7) / 8) * n_second * XRUN;
+}
+
 // ------------------------------------------------------------------ plan
 __global__ __launch_bounds__(1024) void sgmv_plan_kernel(const SgmvArgs p)
 {
@@ -147,7 +169,8 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
     constexpr int AP = (RMAX * CPR + SG_NT - 1) / SG_NT;   // A loads per thread and stage (1, 2 or 4)
     __shared__ __attribute__((aligned(16))) unsigned char s_x[TM * PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char s_a[RMAX * PITCH];
-    const int tile = blockIdx.x, split = blockIdx.y;
+    int tile, split;
+    xcd_remap(blockIdx.x, p.ksplit, tile, split);
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1];
@@ -273,7 +296,7 @@ __global__ __launch_bounds__(256) void sgmv_reduce_kernel(const SgmvArgs p)
 
 // ------------------------------------------------------------------ expand
 template <int DT, int RMAX, bool BT>
-__global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, int cols_per_block)
+__global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, int cols_per_block, int n_colblk)
 {
     // One workgroup: 64 tokens (16 per wavefront) x cols_per_block output columns, 128 columns per step.
     // The B tile of a step is parked in LDS row-major and read back column-wise with the transposing LDS
@@ -293,7 +316,8 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     typedef __attribute__((address_space(3))) volatile float lds_vfloat;
     typedef __attribute__((address_space(3))) volatile float4_t lds_vfloat4;
 
-    const int tile = blockIdx.x;
+    int tile, colblk;
+    xcd_remap(blockIdx.x, n_colblk, tile, colblk);
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1], r = rec[2];
@@ -305,7 +329,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 15, g = lane >> 4;
-    const int col_begin = blockIdx.y * cols_per_block;
+    const int col_begin = colblk * cols_per_block;
     int col_end = col_begin + cols_per_block;
     col_end = col_end < hout ? col_end : hout;
 
@@ -460,7 +484,7 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
         if (rc) return rc;
     }
     if (!(phases & SGMV_APPLY)) return 0;
-    hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3(a.max_tiles, a.ksplit), dim3(SG_NT), 0, s, a);
+    hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3((unsigned)xcd_grid(a.max_tiles, a.ksplit)), dim3(SG_NT), 0, s, a);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     {
@@ -473,10 +497,11 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
     int cols = 512;
     while (cols > TN && (long long)a.max_tiles * ((a.hout + cols - 1) / cols) < 1024) cols >>= 1;
     const int ncb = (a.hout + cols - 1) / cols;
+    const unsigned egrid = (unsigned)xcd_grid(a.max_tiles, ncb);
     if (a.b_transposed)
-        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, true>), dim3(a.max_tiles, ncb), dim3(SG_NT), 0, s, a, cols);
+        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, true>), dim3(egrid), dim3(SG_NT), 0, s, a, cols, ncb);
     else
-        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, false>), dim3(a.max_tiles, ncb), dim3(SG_NT), 0, s, a, cols);
+        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, false>), dim3(egrid), dim3(SG_NT), 0, s, a, cols, ncb);
     return (int)hipGetLastError();
 }
 
