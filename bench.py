@@ -27,6 +27,11 @@ for _p in (ROOT, os.path.join(ROOT, "ae-296_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per BGMV launch of the default workload, from the two counter runs summarised in
+# profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
+# same runs).  Reported as roofline.traffic only when the run is that same configuration.
+MEASURED_TRAFFIC_C2 = 81.28e6
+MEASURED_TRAFFIC_C4_STEP = 3326.5e6
 
 
 def log(*a):
@@ -117,7 +122,7 @@ def bench_c4(args, dev):
            "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
                                   "32 rank-64 adapters, bf16", "tokens": T, "segments": 16},
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                        "traffic": None, "kernel": "sgmv plan+shrink+reduce+expand, 7 projections",
+                        "traffic": MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)",
                         "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
            "cpu_baseline": None}
     print(json.dumps(out), flush=True)
@@ -238,7 +243,8 @@ def main():
                    "tokens": T, "adapters": 64, "adapters_touched": int(len(uniq)), "group": args.group,
                    "hip_graph": not args.no_graph, "wall_s_timed_region": wall},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_C2 if (args.group == 4 and L == 32) else None,
                      "kernel": "bgmv_kernel (4 projections per launch)", "launch_us": launch_us,
                      "algorithmic_bytes_per_launch": alg, "per_token_gather_bytes_per_launch": per_token_gather},
         "cpu_baseline": None,
