@@ -67,8 +67,8 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
         // Records are stored in launch order: record b belongs to workgroup b of every projection.
         // The gather interleaves consecutive chunks over the 8 XCDs (workgroups are dealt to XCDs
         // round-robin by id), so the chunks of one hot adapter share one XCD's L2.
-        const int b = blockIdx.x % p.work_cap;
-        proj = blockIdx.x / p.work_cap;
+        const int b = blockIdx.x % p.items_cap;
+        proj = blockIdx.x / p.items_cap;
         const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
         ntok = rec[0];
         if (ntok <= 0) return;
@@ -361,7 +361,7 @@ template <int DT, int G, int RMAX, bool BT, bool WORK>
 static int launch_one(const BgmvArgs &a, hipStream_t s)
 {
     constexpr int NT = 256;
-    const long long per_proj = WORK ? a.work_cap : a.T;
+    const long long per_proj = WORK ? a.items_cap : a.T;
     const long long total = (long long)a.n_proj * per_proj;
     if (total <= 0) return 0;
     if (total > 0x7fffffffLL) return (int)hipErrorInvalidValue;

@@ -1,0 +1,307 @@
+// BGMV decode as two launches for gfx950: a shrink launch that writes x . A as fp32 partial sums
+// per slice of the Hin columns, and an expand launch that sums the slices, scales and applies B.
+//
+// Why two launches when one can keep the intermediate on chip: a compute unit can only keep a
+// limited number of cache-line fills in flight, so the chip reaches its memory bandwidth only
+// while every compute unit is pulling data.  The fused kernel's unit of work is a whole item
+// (an adapter's A and B rows for one projection, hundreds of KiB) and a decode batch has about
+// one item per compute unit, so a unit that gets two items finishes late and the others idle.
+// Here the unit of work is a 1024-column slice of an item (tens of KiB), there are several
+// slices per compute unit and per phase, and no row is fetched by more than one workgroup.
+// The price is the intermediate (T x slices x rank fp32, a few hundred KiB) going through L2.
+//
+// Both kernels read the work records the gather wrote (one 320-byte record per item: tokens,
+// adapter, rank, scaling, the row of every rank row).  Workgroup ids enumerate records in units
+// of eight (one per XCD) with the slices and projections of those eight in between, so the
+// records in use come first in launch order and the empty tail costs no waiting.
+//
+// Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
+#include "mlora_args.hpp"
+#include "mlora_dev.hpp"
+
+namespace mlora {
+
+constexpr int SLICE_CHUNKS = 128;                // 16-byte chunks per slice = 1024 columns
+
+struct ItemId { int b, q; };
+
+__device__ __forceinline__ ItemId split_id(unsigned id, int nq)
+{
+    const int g = (int)(id >> 3);
+    ItemId r;
+    r.q = g % nq;
+    r.b = (g / nq) * 8 + (int)(id & 7u);
+    return r;
+}
+
+template <int DT, int G, int RMAX>
+__global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
+{
+    constexpr int NW = 4;
+    constexpr int RPG = RMAX / 4;                               // rank rows per 16-lane row
+    constexpr int U = (RPG + G) <= 12 ? 2 : 1;                  // column steps kept in flight
+    __shared__ float s_part[NW][G][RMAX];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int cl = lane & 15, rg = lane >> 4;
+    const PoolView &pv = p.pool;
+
+    const ItemId id = split_id(blockIdx.x, p.n_proj * p.ks_max);
+    const int proj = id.q / p.ks_max, ks = id.q - proj * p.ks_max;
+    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
+    int ntok = rec[0];
+    if (ntok <= 0) return;
+    ntok = ntok < G ? ntok : G;
+    const int adapter = rec[1];
+    if (adapter < 0) return;
+    const int hin = p.hin[proj];
+    const int ncc_in = hin >> 3;
+    const int kc0 = ks * SLICE_CHUNKS;
+    if (kc0 >= ncc_in) return;                                  // this projection has fewer slices
+    int r = rec[2];
+    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
+    int tok[G];
+#pragma unroll
+    for (int k = 0; k < G; k++) {
+        const int t = k < ntok ? rec[4 + k] : -1;
+        tok[k] = (t >= 0 && t < p.T) ? t : -1;
+    }
+    const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+
+    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x[proj]);
+    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows[proj]);
+
+    // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot beyond
+    // ntok reads token 0 (both discarded below); a chunk past the end of the row re-reads the
+    // last chunk with x forced to zero.
+    const uint4 *ap[RPG];
+    unsigned row_ok = 0;
+#pragma unroll
+    for (int i = 0; i < RPG; i++) {
+        int row = rows[rg + 4 * i];
+        row = (row >= 0 && row < pv.n_rows_a) ? row : -1;
+        row_ok |= (row >= 0 ? 1u : 0u) << i;
+        ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+    }
+    const uint4 *xp[G];
+#pragma unroll
+    for (int k = 0; k < G; k++) xp[k] = reinterpret_cast<const uint4 *>(x + (size_t)(tok[k] >= 0 ? tok[k] : 0) * hin);
+    float acc[G][RPG];
+#pragma unroll
+    for (int k = 0; k < G; k++)
+#pragma unroll
+        for (int i = 0; i < RPG; i++) acc[k][i] = 0.f;
+
+    // Each wavefront covers 32 chunks of the slice: two steps of 16 chunks per 16-lane row.
+#pragma unroll
+    for (int it0 = 0; it0 < 2; it0 += U) {
+        uint4 xv[G][U];
+        uint4 av[RPG][U];
+        bool cv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = kc0 + wave * 32 + (it0 + u) * 16 + cl;
+            cv[u] = c < ncc_in;
+            const int cs = c < ncc_in ? c : ncc_in - 1;
+#pragma unroll
+            for (int k = 0; k < G; k++) xv[k][u] = xp[k][cs];
+#pragma unroll
+            for (int i = 0; i < RPG; i++) av[i][u] = ap[i][cs];
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int k = 0; k < G; k++) {
+                xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
+                xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
+            }
+#pragma unroll
+            for (int i = 0; i < RPG; i++)
+#pragma unroll
+                for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
+        }
+    }
+
+#pragma unroll
+    for (int k = 0; k < G; k++)
+#pragma unroll
+        for (int i = 0; i < RPG; i++) {
+            const float a = ((row_ok >> i) & 1u) ? acc[k][i] : 0.f;
+            const float s = row16_sum(a);
+            if (cl == 0) s_part[wave][k][rg + 4 * i] = s;
+        }
+    __syncthreads();
+    for (int e = tid; e < G * RMAX; e += 256) {
+        const int k = e / RMAX, j = e - k * RMAX;
+        if (j < r && tok[k] >= 0) {
+            float s = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; wv++) s += s_part[wv][k][j];
+            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + ks) * RMAX + j] = s;
+        }
+    }
+}
+
+template <int DT, int G, int RMAX>
+__global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
+{
+    constexpr int NT = 128;                                     // one 16-byte chunk of the slice per thread
+    constexpr int EB = RMAX < 16 ? RMAX : 16;                   // B rank rows in flight per lane
+    __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
+
+    const int tid = threadIdx.x;
+    const PoolView &pv = p.pool;
+
+    const ItemId id = split_id(blockIdx.x, p.n_proj * p.cs_max);
+    const int proj = id.q / p.cs_max, cs = id.q - proj * p.cs_max;
+    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
+    int ntok = rec[0];
+    if (ntok <= 0) return;
+    ntok = ntok < G ? ntok : G;
+    const int hout = p.hout[proj];
+    const int ncc_out = hout >> 3;
+    if (cs * SLICE_CHUNKS >= ncc_out) return;                   // this projection has fewer slices
+    const int cc = cs * SLICE_CHUNKS + tid;
+    const bool active = cc < ncc_out;
+    const int adapter = rec[1];
+    int r = rec[2];
+    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
+    const float scale = __builtin_bit_cast(float, rec[3]);
+    int tok[G];
+#pragma unroll
+    for (int k = 0; k < G; k++) {
+        const int t = k < ntok ? rec[4 + k] : -1;
+        tok[k] = (t >= 0 && t < p.T) ? t : -1;
+    }
+    const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+    uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y[proj]);
+    const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(p.b_rows[proj]);
+
+    if (adapter < 0) {
+        if (!p.accumulate && active) {
+#pragma unroll
+            for (int k = 0; k < G; k++)
+                if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, zero16());
+        }
+        return;
+    }
+
+    auto b_rows_of = [&](int j0, int (&out)[EB]) {              // rows of rank rows j0 .. j0+EB-1
+        if constexpr (EB % 4 == 0) {
+            const int4 *q = reinterpret_cast<const int4 *>(rows + j0);
+#pragma unroll
+            for (int m = 0; m < EB / 4; m++) {
+                const int4 v = q[m];
+                out[4 * m] = v.x; out[4 * m + 1] = v.y; out[4 * m + 2] = v.z; out[4 * m + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++) out[jj] = rows[j0 + jj];
+        }
+#pragma unroll
+        for (int jj = 0; jj < EB; jj++) out[jj] = (out[jj] >= 0 && out[jj] < pv.n_rows_b) ? out[jj] : -1;
+    };
+
+    // Everything the first step needs is requested before the partial sums are fetched.
+    uint4 bv[EB];
+    uint4 yv[G];
+    if (active) {
+        int br[EB];
+        b_rows_of(0, br);
+#pragma unroll
+        for (int jj = 0; jj < EB; jj++)
+            bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+#pragma unroll
+        for (int k = 0; k < G; k++)
+            yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
+    }
+
+    // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
+    const int n_ks = ((p.hin[proj] >> 3) + SLICE_CHUNKS - 1) / SLICE_CHUNKS;
+    for (int e = tid; e < G * RMAX; e += NT) {
+        const int k = e / RMAX, j = e - k * RMAX;
+        float s = 0.f;
+        if (j < r && tok[k] >= 0) {
+            const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
+            for (int ks = 0; ks < n_ks; ks++) s += src[(size_t)ks * RMAX];
+        }
+        s_v[k][j] = s * scale;
+    }
+    __syncthreads();
+    if (!active) return;
+
+    float o[G][8];
+#pragma unroll
+    for (int k = 0; k < G; k++) unpack8<DT>(yv[k], o[k]);
+#pragma unroll 1
+    for (int j0 = 0; j0 < r; j0 += EB) {
+        if (j0 > 0) {
+            int br[EB];
+            b_rows_of(j0, br);
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++)
+                bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+        }
+#pragma unroll
+        for (int jj = 0; jj < EB; jj++) {
+            float f[8];
+            unpack8<DT>(bv[jj], f);
+#pragma unroll
+            for (int k = 0; k < G; k++) {
+                const float vk = s_v[k][j0 + jj];
+#pragma unroll
+                for (int e = 0; e < 8; e++) o[k][e] = fmaf(vk, f[e], o[k][e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < G; k++)
+        if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
+}
+
+template <int DT, int G, int RMAX>
+static int launch_pair(const BgmvArgs &a, hipStream_t s)
+{
+    const long long n_sh = (long long)a.n_proj * a.ks_max * a.items_cap;
+    const long long n_ex = (long long)a.n_proj * a.cs_max * a.items_cap;
+    if (n_sh <= 0 || n_ex <= 0) return 0;
+    if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL((bgmv_expand_kernel<DT, G, RMAX>), dim3((unsigned)n_ex), dim3(128), 0, s, a);
+    return (int)hipGetLastError();
+}
+
+template <int DT, int RMAX>
+static int launch_group(const BgmvArgs &a, int group, hipStream_t s)
+{
+    switch (group) {
+    case 1: return launch_pair<DT, 1, RMAX>(a, s);
+    case 2: return launch_pair<DT, 2, RMAX>(a, s);
+    case 4: return launch_pair<DT, 4, RMAX>(a, s);
+    case 8:
+        if constexpr (RMAX <= 32) return launch_pair<DT, 8, RMAX>(a, s);
+        else return (int)hipErrorInvalidValue;
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
+template <int DT>
+static int launch_split_dt(const BgmvArgs &a, int group, int max_rank, hipStream_t s)
+{
+    if (max_rank <= 16) return launch_group<DT, 16>(a, group, s);
+    if (max_rank <= 32) return launch_group<DT, 32>(a, group, s);
+    return launch_group<DT, 64>(a, group, s);
+}
+
+int bgmv_split_rank_stride(int max_rank) { return max_rank <= 16 ? 16 : (max_rank <= 32 ? 32 : 64); }
+
+int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s)
+{
+    if (!a.work || !a.vws) return (int)hipErrorInvalidValue;
+    if (dtype == DT_F16) return launch_split_dt<DT_F16>(a, group, max_rank, s);
+    return launch_split_dt<DT_BF16>(a, group, max_rank, s);
+}
+
+}  // namespace mlora

@@ -110,11 +110,19 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
     return MLORA_OK;
 }
 
+int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
+{
+    if (n_proj < 1 || T < 1 || max_hin < 1) return 0;
+    const int64_t ks = (max_hin + 1023) / 1024;
+    return (int64_t)n_proj * T * ks * mlora::bgmv_split_rank_stride(max_rank) * (int64_t)sizeof(float);
+}
+
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
                      const void *const *b_rows, const int32_t *hin, const int32_t *hout,
                      const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
                      const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
-                     int max_rank, const int32_t *work, int group, int dtype, int accumulate, void *stream)
+                     int max_rank, const int32_t *work, int group, void *workspace, int64_t workspace_bytes,
+                     int dtype, int accumulate, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
@@ -133,6 +141,8 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
     } else if (group != 1) {
         return fail(MLORA_EINVAL, "group must be 1 when work is NULL (got %d)", group);
     }
+    if (workspace && !work) return fail(MLORA_EINVAL, "the two-launch form (workspace given) needs the work records");
+    int max_hin = 0, max_hout = 0;
     for (int p = 0; p < n_proj; p++) {
         if (!y[p] || !x[p] || !a_rows[p] || !b_rows[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
         if (!aligned16(y[p]) || !aligned16(x[p]) || !aligned16(a_rows[p]) || !aligned16(b_rows[p]))
@@ -141,11 +151,32 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
         if (rc) return rc;
         a.y[p] = y[p]; a.x[p] = x[p]; a.a_rows[p] = a_rows[p]; a.b_rows[p] = b_rows[p];
         a.hin[p] = hin[p]; a.hout[p] = hout[p];
+        max_hin = hin[p] > max_hin ? hin[p] : max_hin;
+        max_hout = hout[p] > max_hout ? hout[p] : max_hout;
     }
     a.tok_adapter = tok_adapter; a.tok_adapter64 = nullptr;
     a.work = work; a.work_cap = MLORA_WORK_CAP(T);
+    {
+        // Work items in use <= T/group + segments + 1 (one short piece per adapter present, one for the
+        // adapter-less tokens); the gather packs them into the first records, so the rest needs no workgroup.
+        const int g = group > 0 ? group : 1;
+        const int64_t segs = T < n_adapters ? T : n_adapters;
+        const int64_t bound = ((int64_t)(T + g - 1) / g + segs + 1 + 7) / 8 * 8;
+        a.items_cap = bound < a.work_cap ? (int)bound : a.work_cap;
+    }
     a.T = T; a.n_proj = n_proj; a.accumulate = accumulate ? 1 : 0;
-    rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));
+    if (workspace) {
+        const int64_t need = mlora_bgmv_workspace_bytes(n_proj, T, max_hin, max_rank);
+        if (workspace_bytes < need)
+            return fail(MLORA_ENOSPACE, "workspace holds %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+        if (!aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be 16-byte aligned");
+        a.vws = static_cast<float *>(workspace);
+        a.ks_max = (max_hin + 1023) / 1024;
+        a.cs_max = (max_hout + 1023) / 1024;
+        rc = mlora::launch_bgmv_split(a, dtype, group, max_rank, static_cast<hipStream_t>(stream));
+    } else {
+        rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));
+    }
     if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
 }
@@ -159,7 +190,7 @@ int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows, c
     const void *xs[1] = {x}, *as[1] = {a_rows}, *bs[1] = {b_rows};
     const int32_t hi[1] = {hin}, ho[1] = {hout};
     return mlora_bgmv_multi(1, ys, xs, as, bs, hi, ho, tok_adapter, T, page_tbl, rank, scaling, n_adapters,
-                            max_pages, page_rows, n_pages, max_rank, nullptr, 1, dtype, accumulate, stream);
+                            max_pages, page_rows, n_pages, max_rank, nullptr, 1, nullptr, 0, dtype, accumulate, stream);
 }
 
 int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const void *wb_T_all,

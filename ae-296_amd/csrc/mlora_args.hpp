@@ -45,10 +45,14 @@ struct BgmvArgs {
     const int32_t *tok_adapter;    // [T] int32, or nullptr when tok_adapter64 is used
     const int64_t *tok_adapter64;  // [T] int64 (reference layout call)
     const int32_t *work;           // work records in launch order (nullptr => one token per workgroup)
-    int work_cap;                  // records (= workgroups per projection), a multiple of 8
+    int work_cap;                  // records the gather wrote (in use or empty), a multiple of 8
+    int items_cap;                 // records that can be in use for this T, group and pool (<= work_cap, multiple of 8)
     int T;
     int n_proj;
     int accumulate;
+    float *vws;                    // two-launch form: partial sums [n_proj, T, ks_max, rank stride] (else nullptr)
+    int ks_max;                    // 1024-column slices of the widest hin
+    int cs_max;                    // 1024-column slices of the widest hout
 };
 
 struct GatherArgs {
@@ -97,6 +101,8 @@ struct SgmvArgs {
 
 // launchers (defined next to their kernels); return hipError_t as int
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
+int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);
+int bgmv_split_rank_stride(int max_rank);
 int launch_gather(const GatherArgs &a, hipStream_t s);
 constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
 constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)

@@ -81,7 +81,18 @@ __device__ __forceinline__ uint32_t cvt16(float f)
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi)
 {
-    return cvt16<DT>(lo) | (cvt16<DT>(hi) << 16);
+    if constexpr (DT == DT_F16) {
+        // Converted as a pair (v_cvt_pk_f16_f32).  A scalar conversion can be folded by the compiler
+        // into the last multiply-add of a chain (v_fma_mixlo_f16), which rounds the exact sum to 16
+        // bits in one step; it does so for some outputs and not for others, so results would depend
+        // on register allocation.  Every output is rounded fp32 -> fp16 here.
+        typedef float f32x2 __attribute__((ext_vector_type(2)));
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    } else {
+        return cvt16<DT>(lo) | (cvt16<DT>(hi) << 16);
+    }
 }
 
 template <int DT>

@@ -37,8 +37,9 @@ SIGNATURES = {
     "mlora_version": (_i32, []),
     "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+    "mlora_bgmv_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
-                                _i64, _i32, _vp, _i32, _i32, _i32, _vp]),
+                                _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),
     "mlora_bgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i64,
                           _i32, _i32, _i32, _vp]),
     "mlora_bgmv_reflayout": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),

@@ -57,6 +57,7 @@ class DecodePlan:
     row_off: Optional[torch.Tensor] = None   # int32 [T, max_pages]
     tok_rank: Optional[torch.Tensor] = None
     tok_scale: Optional[torch.Tensor] = None
+    vws: Optional[torch.Tensor] = None       # uint8: fp32 intermediate of the two-launch decode form
 
     @property
     def T(self) -> int:
@@ -104,9 +105,15 @@ def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: int = 4, pe
 # ---------------------------------------------------------------------- decode
 def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPool, layer: int,
          projs: Sequence[str], tok_adapter: torch.Tensor, plan: Optional[DecodePlan] = None,
-         accumulate: bool = True) -> None:
-    """Decode LoRA apply for up to 8 projections of one layer in one launch:
-    ys[p][t] (+)= scaling[a] * (xs[p][t] . A_{p,a}) . B_{p,a},  a = tok_adapter[t]."""
+         accumulate: bool = True, fused: Optional[bool] = None) -> None:
+    """Decode LoRA apply for up to 8 projections of one layer:
+    ys[p][t] (+)= scaling[a] * (xs[p][t] . A_{p,a}) . B_{p,a},  a = tok_adapter[t].
+
+    With a plan the call runs as a shrink launch and an expand launch over column slices
+    (``fused=False``, the default) or as one fused launch (``fused=True``); without a plan it is
+    always the fused launch with one token per work item.  The two-launch form keeps its fp32
+    intermediate in a buffer owned by the plan, allocated on the first call that needs it (so
+    run one call before capturing a HIP graph)."""
     n = len(projs)
     if not (len(ys) == len(xs) == n) or not 1 <= n <= _ext.MAX_PROJ:
         raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y and one x each")
@@ -128,11 +135,22 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     pool.sync()
     if plan is not None and plan.T != T:
         raise ValueError("plan was built for a different batch size")
+    if fused is None:
+        fused = plan is None
+    if not fused and plan is None:
+        raise ValueError("the two-launch form needs a plan")
+    ws, ws_bytes = None, 0
+    if not fused:
+        ws_bytes = _ext.lib().mlora_bgmv_workspace_bytes(n, T, max(hi[i] for i in range(n)), pool.max_rank)
+        if plan.vws is None or plan.vws.numel() < ws_bytes:
+            plan.vws = torch.empty(ws_bytes, dtype=torch.uint8, device=tok_adapter.device)
+        ws = plan.vws
     rc = _ext.lib().mlora_bgmv_multi(
         n, yv, xv, av, bv, hi, ho, _ext.ptr(tok_adapter), T,
         _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
         pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.max_rank,
         _ext.ptr(plan.work) if plan else None, plan.group if plan else 1,
+        _ext.ptr(ws), ws_bytes,
         pool.dtype_code, int(accumulate), _ext.current_stream_ptr())
     _ext.check(rc)
 

@@ -4,13 +4,14 @@
 Workload (the configuration the metric is quoted on): decode BGMV over the Llama-7B attention
 projections q/k/v/o (4096 -> 4096 each), 256 decode tokens, 64 rank-16 fp16 adapters in one paged
 pool, adapter per token ~ Zipf(1.0), scaling 2.0.  One step = one decode step's LoRA work: the
-adapter-pool gather once, then for each of the 32 layers one fused BGMV launch covering that
-layer's q, k, v (shared input) and o (own input), accumulating into the base projection outputs.
+adapter-pool gather once, then for each of the 32 layers one BGMV call (a shrink launch and an
+expand launch, or one fused launch with --fused) covering that layer's q, k, v (shared input) and
+o (own input), accumulating into the base projection outputs.
 Every layer has its own pool slabs, inputs and outputs (about 2.4 GB in all), so a step streams
 from HBM rather than from the 256 MB last-level cache.
 
-Prints one JSON line: throughput in token-projections/s, the HBM roofline of the BGMV kernel
-(algorithmic bytes / measured launch duration) and the CPU baseline (the CPU-assisted path's
+Prints one JSON line: throughput in token-projections/s, the HBM roofline of the BGMV call
+(algorithmic bytes / measured duration of one layer's launches) and the CPU baseline (the CPU-assisted path's
 arithmetic timed on the host cores).
 """
 from __future__ import annotations
@@ -135,6 +136,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
+    ap.add_argument("--fused", action="store_true", help="one fused launch per layer instead of the shrink + expand pair")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
@@ -179,10 +181,11 @@ def main():
     x_o = [torch.randn(T, 4096, device=dev, generator=gen).half() for _ in range(L)]
     ys = [[torch.randn(T, 4096, device=dev, generator=gen).half() for _ in projs] for _ in range(L)]
     plan = mlora.plan_decode(tok, pool, group=args.group) if args.group else None
+    fused = bool(args.fused or plan is None)
 
     def bgmv_layers():
         for l in range(L):
-            mlora.bgmv(ys[l], [x_qkv[l], x_qkv[l], x_qkv[l], x_o[l]], pool, l, projs, tok, plan=plan)
+            mlora.bgmv(ys[l], [x_qkv[l], x_qkv[l], x_qkv[l], x_o[l]], pool, l, projs, tok, plan=plan, fused=fused)
 
     def step():
         if plan is not None:
@@ -220,7 +223,7 @@ def main():
     ms_per_step = ms / args.steps
     value = T * len(projs) * L / (ms_per_step * 1e-3)
 
-    # The dominant kernel alone: the same 32 launches without the gather, for the roofline figure.
+    # The BGMV calls alone: the same 32 layers without the gather, for the roofline figure.
     run_bgmv = make_runner(bgmv_layers)
     for _ in range(args.warmup):
         run_bgmv()
@@ -239,13 +242,16 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config 2: decode BGMV, Llama-7B q/k/v/o 4096->4096, 256 tokens, 64 rank-16 adapters, "
                                "Zipf(1.0), fp16, scaling 2.0",
-                   "layers": L, "projections_per_launch": len(projs), "launches_per_step": L + (1 if plan else 0),
+                   "layers": L, "projections_per_launch": len(projs), "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0),
+                   "form": "fused" if fused else "shrink + expand",
                    "tokens": T, "adapters": 64, "adapters_touched": int(len(uniq)), "group": args.group,
                    "hip_graph": not args.no_graph, "wall_s_timed_region": wall},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_C2 if (args.group == 4 and L == 32) else None,
-                     "kernel": "bgmv_kernel (4 projections per launch)", "launch_us": launch_us,
+                     "traffic": MEASURED_TRAFFIC_C2 if (args.group == 4 and L == 32 and not fused) else None,
+                     "kernel": "bgmv_kernel (4 projections per launch)" if fused else
+                               "bgmv_shrink_kernel + bgmv_expand_kernel (one layer's pair, 4 projections)",
+                     "launch_us": launch_us,
                      "algorithmic_bytes_per_launch": alg, "per_token_gather_bytes_per_launch": per_token_gather},
         "cpu_baseline": None,
     }

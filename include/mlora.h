@@ -121,7 +121,14 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T,
  * same `group` (1, 2, 4 or 8; 8 needs max_rank <= 32); tokens of one adapter then share one read
  * of its rows and each workgroup starts from one record instead of walking the tables.
  * With work == NULL every token is its own work item and group must be 1.
+ * Two-launch form: with a `workspace` of mlora_bgmv_workspace_bytes(n_proj, T, max hin, max_rank)
+ * bytes (and work records) the call runs as a shrink launch and an expand launch over
+ * 1024-column slices of the items, the fp32 intermediate passing through the workspace; on a
+ * decode batch with about one item per compute unit this balances the load far better than the
+ * fused launch.  workspace == NULL selects the fused launch.  Both forms accumulate in fp32 and
+ * round once; they differ only in the order the fp32 partial sums of the shrink are added.
  */
+int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank);
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
                      const void *const *a_rows, const void *const *b_rows,
                      const int32_t *hin, const int32_t *hout,
@@ -129,6 +136,7 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
                      const int32_t *page_tbl, const int32_t *rank, const float *scaling,
                      int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
                      const int32_t *work, int group,
+                     void *workspace, int64_t workspace_bytes,
                      int dtype, int accumulate, void *stream);
 
 /* One projection, one token per work item: the plain form of the call above. */

@@ -43,11 +43,11 @@ def test_validation_errors_without_gpu():
 
     def bgmv(**kw):
         a = dict(n_proj=1, hin=H, T=4, n_adapters=4, max_pages=8, page_rows=8, n_pages=10, max_rank=64, work=None,
-                 group=1, dtype=0, y=P)
+                 group=1, dtype=0, y=P, ws=None, ws_bytes=0)
         a.update(kw)
         return lib.mlora_bgmv_multi(a["n_proj"], a["y"], P, P, P, a["hin"], H, one, a["T"], one, one, one,
                                     a["n_adapters"], a["max_pages"], a["page_rows"], a["n_pages"], a["max_rank"],
-                                    a["work"], a["group"], a["dtype"], 1, None)
+                                    a["work"], a["group"], a["ws"], a["ws_bytes"], a["dtype"], 1, None)
 
     assert bgmv(T=0) == _ext.MLORA_OK
     assert bgmv(dtype=7) == _ext.MLORA_EDTYPE
@@ -55,6 +55,11 @@ def test_validation_errors_without_gpu():
     assert bgmv(n_proj=9) == _ext.MLORA_ERANGE
     assert bgmv(max_rank=65) == _ext.MLORA_ERANGE
     assert bgmv(page_rows=3) == _ext.MLORA_EINVAL
+    assert bgmv(ws=16, ws_bytes=1 << 20) == _ext.MLORA_EINVAL            # two-launch form without work records
+    assert b"work records" in lib.mlora_last_error()
+    assert bgmv(ws=16, ws_bytes=64, work=16, group=4) == _ext.MLORA_ENOSPACE
+    assert lib.mlora_bgmv_workspace_bytes(4, 256, 4096, 16) == 4 * 256 * 4 * 16 * 4
+    assert lib.mlora_bgmv_workspace_bytes(1, 10, 11008, 33) == 10 * 11 * 64 * 4
     assert bgmv(max_pages=1, page_rows=8, max_rank=16) == _ext.MLORA_ERANGE
     assert bgmv(hin=(C.c_int32 * 8)(60, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
     assert bgmv(y=(C.c_void_p * 8)(8, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN

@@ -1,5 +1,6 @@
-"""GPU parity: fused BGMV decode kernel through the C ABI against the fp32-accumulated oracle
-(rtol 1e-2 / atol 1e-3), on seeded inputs, plus size-independent properties at full size."""
+"""GPU parity: BGMV decode through the C ABI, fused launch and shrink + expand pair, against the
+fp32-accumulated oracle (rtol 1e-2 / atol 1e-3), on seeded inputs, plus size-independent
+properties at full size."""
 import zlib
 
 import numpy as np
@@ -18,16 +19,20 @@ def _zipf(rng, T, N, alpha):
     return rng.permutation(N)[rng.choice(N, size=T, p=p / p.sum())].astype(np.int32)
 
 
-def _run(pp, x_bits, tok, y0_bits, group, accumulate=True):
+def _run(pp, x_bits, tok, y0_bits, group, accumulate=True, fused=None):
     pool = upload_pool(pp)
     x = bits_to_torch(x_bits, pp.dtype, "cuda")
     y = bits_to_torch(y0_bits, pp.dtype, "cuda") if y0_bits is not None else \
         torch.full((len(tok), pp.hout), float("nan"), dtype=tdtype(pp.dtype), device="cuda")
     t = torch.from_numpy(tok).cuda()
     plan = plan_decode(t, pool, group=group) if group > 0 else None
-    bgmv([y], [x], pool, 0, ["p"], t, plan=plan, accumulate=accumulate)
+    bgmv([y], [x], pool, 0, ["p"], t, plan=plan, accumulate=accumulate, fused=fused)
     torch.cuda.synchronize()
     return torch_to_bits(y)
+
+
+# launch forms: (group, fused); group 0 = no plan, one token per work item
+FORMS = [(0, True), (1, True), (4, True), (1, False), (2, False), (4, False)]
 
 
 CASES = [
@@ -63,21 +68,21 @@ def _case(name):
 
 
 @pytest.mark.parametrize("name", [c[0] for c in CASES])
-@pytest.mark.parametrize("group", [0, 1, 4])
-def test_bgmv_vs_oracle(name, group):
+@pytest.mark.parametrize("group,fused", FORMS)
+def test_bgmv_vs_oracle(name, group, fused):
     dtype = next(c for c in CASES if c[0] == name)[6]
     pp, tok, x, y0, want, want_d = _case(name)
-    say(f"bgmv {name} group={group} accumulate")
-    got = _run(pp, x, tok, y0, group)
+    say(f"bgmv {name} group={group} fused={fused} accumulate")
+    got = _run(pp, x, tok, y0, group, fused=fused)
     assert_close_bits(got, want, dtype, name)
     # the delta alone must also meet the tolerance (y = delta form, reference's zeros+bgmv at lora_gpu.py:137-138)
-    say(f"bgmv {name} group={group} delta")
-    got_d = _run(pp, x, tok, None, group, accumulate=False)
+    say(f"bgmv {name} group={group} fused={fused} delta")
+    got_d = _run(pp, x, tok, None, group, accumulate=False, fused=fused)
     assert_close_bits(got_d, want_d, dtype, name + " delta")
 
 
-@pytest.mark.parametrize("group", [0, 2, 8])
-def test_bgmv_integer_inputs_bit_exact(group):
+@pytest.mark.parametrize("group,fused", [(0, True), (2, True), (8, True), (1, False), (2, False), (8, False)])
+def test_bgmv_integer_inputs_bit_exact(group, fused):
     """Integer-valued inputs make every fp32 operation exact: the kernel must match bit for bit."""
     rng = np.random.default_rng(41)
     ranks = [8, 16, 3, 1, 5, 32]
@@ -91,8 +96,8 @@ def test_bgmv_integer_inputs_bit_exact(group):
     x = bits_of(xi, FP16)
     want = oracle_apply(pp, x, tok, y0)
     assert np.abs(f32_of(want, FP16)).max() < 2048
-    say(f"bgmv integer-valued inputs group={group}")
-    got = _run(pp, x, tok, y0, group)
+    say(f"bgmv integer-valued inputs group={group} fused={fused}")
+    got = _run(pp, x, tok, y0, group, fused=fused)
     assert np.array_equal(got, want)
 
 
@@ -104,12 +109,12 @@ def test_bgmv_tokens_without_adapter_and_rank_tails():
     tok[:3] = -1
     x = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
     y0 = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
-    for group in (0, 4):
-        say(f"bgmv no-adapter tokens group={group}")
-        got = _run(pp, x, tok, y0, group)
+    for group, fused in ((0, True), (4, True), (4, False), (2, False)):
+        say(f"bgmv no-adapter tokens group={group} fused={fused}")
+        got = _run(pp, x, tok, y0, group, fused=fused)
         assert np.array_equal(got[tok < 0], y0[tok < 0])          # untouched, bit for bit
         assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16)
-        got_d = _run(pp, x, tok, None, group, accumulate=False)
+        got_d = _run(pp, x, tok, None, group, accumulate=False, fused=fused)
         assert np.all(got_d[tok < 0] == 0)                        # y = delta defines those rows as zero
         assert_close_bits(got_d, oracle_apply(pp, x, tok, None), FP16)
 
@@ -136,12 +141,14 @@ def test_bgmv_multi_projection_one_launch():
     xs = {p: bits_to_torch(x_o if p == "o" else x_qkv, FP16, "cuda") for p in "qkvo"}
     ys = {p: bits_to_torch(y0[p], FP16, "cuda") for p in "qkvo"}
     plan = plan_decode(t, pool, group=4)
-    say("bgmv 4 projections in one launch")
-    bgmv([ys[p] for p in "qkvo"], [xs[p] for p in "qkvo"], pool, 0, list("qkvo"), t, plan=plan)
-    torch.cuda.synchronize()
-    for p in "qkvo":
-        want = oracle_apply(pps[p], x_o if p == "o" else x_qkv, tok, y0[p])
-        assert_close_bits(torch_to_bits(ys[p]), want, FP16, f"projection {p}")
+    for fused in (True, False):
+        ys = {p: bits_to_torch(y0[p], FP16, "cuda") for p in "qkvo"}
+        say(f"bgmv 4 projections in one call fused={fused}")
+        bgmv([ys[p] for p in "qkvo"], [xs[p] for p in "qkvo"], pool, 0, list("qkvo"), t, plan=plan, fused=fused)
+        torch.cuda.synchronize()
+        for p in "qkvo":
+            want = oracle_apply(pps[p], x_o if p == "o" else x_qkv, tok, y0[p])
+            assert_close_bits(torch_to_bits(ys[p]), want, FP16, f"projection {p}")
 
 
 def test_bgmv_full_size_properties():
@@ -156,25 +163,30 @@ def test_bgmv_full_size_properties():
     y0 = torch.randn(T, H, device="cuda", dtype=torch.float16)
     t = torch.from_numpy(tok).cuda()
 
-    def run(xx, tt, yy0, group):
+    def run(xx, tt, yy0, group, fused=True):
         y = yy0.clone()
         plan = plan_decode(tt, pool, group=group) if group else None
-        bgmv([y], [xx], pool, 0, ["p"], tt, plan=plan)
+        bgmv([y], [xx], pool, 0, ["p"], tt, plan=plan, fused=fused)
         return y
 
     say("bgmv full-size: direct vs grouped")
     y_direct = run(x, t, y0, 0)
     y_g4 = run(x, t, y0, 4)
     y_g8 = run(x, t, y0, 8)
+    y_s2, y_s4, y_s8 = (run(x, t, y0, g, fused=False) for g in (2, 4, 8))
     torch.cuda.synchronize()
-    for other in (y_g4, y_g8):
+    for other in (y_g4, y_g8, y_s4):
         assert torch.allclose(other.float(), y_direct.float(), rtol=RTOL, atol=ATOL)
-    # a token's result does not depend on which other tokens share its work item: same summation order
+    # a token's result does not depend on which other tokens share its work item: within one launch
+    # form the summation order is fixed, so the results agree bit for bit
     assert torch.equal(y_g4, y_direct) and torch.equal(y_g8, y_direct)
+    assert torch.equal(y_s2, y_s4) and torch.equal(y_s8, y_s4)
     say("bgmv full-size: token permutation")
     perm = torch.randperm(T, device="cuda")
     y_perm = run(x[perm].contiguous(), t[perm].contiguous(), y0[perm].contiguous(), 4)
     assert torch.equal(y_perm, y_g4[perm])
+    y_perm = run(x[perm].contiguous(), t[perm].contiguous(), y0[perm].contiguous(), 4, fused=False)
+    assert torch.equal(y_perm, y_s4[perm])
     say("bgmv full-size: lora_apply")
     y_api = lora_apply(y0.clone(), x, t, pool, 0, "p")
     torch.cuda.synchronize()
@@ -186,9 +198,11 @@ def test_bgmv_full_size_properties():
         pp2.b_rows[pp2.rows(i)] = pp.b_rows[pp.rows(i)]
     pool2 = upload_pool(pp2)
     y2 = y0.clone()
-    bgmv([y2], [x], pool2, 0, ["p"], t, plan=plan_decode(t, pool2, group=4))
+    bgmv([y2], [x], pool2, 0, ["p"], t, plan=plan_decode(t, pool2, group=4), fused=True)
+    y3 = y0.clone()
+    bgmv([y3], [x], pool2, 0, ["p"], t, plan=plan_decode(t, pool2, group=4), fused=False)
     torch.cuda.synchronize()
-    assert torch.equal(y2, y_g4)
+    assert torch.equal(y2, y_g4) and torch.equal(y3, y_s4)
     say("bgmv full-size: linearity of the delta")
     d1 = torch.zeros_like(y0)
     d2 = torch.zeros_like(y0)
