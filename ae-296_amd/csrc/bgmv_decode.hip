@@ -197,9 +197,9 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             cv[u] = (it0 + u) < n_it && c < ncc_in;
             const int cs = c < ncc_in ? c : ncc_in - 1;
 #pragma unroll
-            for (int k = 0; k < G; k++) xv[k][u] = xp[k][cs];
+            for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + cs);
 #pragma unroll
-            for (int i = 0; i < RPG; i++) av[i][u] = ap[i][cs];
+            for (int i = 0; i < RPG; i++) av[i][u] = ldg16_stream(ap[i] + cs);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -224,10 +224,10 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             b_rows_of(0, br);
 #pragma unroll
             for (int jj = 0; jj < EB; jj++)
-                bpre[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)tid * 8) : zero16();
+                bpre[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)tid * 8) : zero16();
 #pragma unroll
             for (int k = 0; k < G; k++)
-                ypre[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)tid * 8) : zero16();
+                ypre[k] = (p.accumulate && tok[k] >= 0) ? ldg16_stream(y + (size_t)tok[k] * hout + (size_t)tid * 8) : zero16();
         }
     }
 
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             for (int k = 0; k < G; k++) {
                 if (p.accumulate && tok[k] >= 0) {
                     uint4 yv;
-                    if (pre) yv = ypre[k]; else yv = ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8);
+                    if (pre) yv = ypre[k]; else yv = ldg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8);
                     unpack8<DT>(yv, o[k]);
                 } else {
 #pragma unroll
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
                     b_rows_of(j0, br);
 #pragma unroll
                     for (int jj = 0; jj < EB; jj++)
-                        bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+                        bv[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
                 }
 #pragma unroll
                 for (int jj = 0; jj < EB; jj++) {
@@ -293,7 +293,7 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
             }
 #pragma unroll
             for (int k = 0; k < G; k++)
-                if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
+                if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
         }
     } else {
         // B given as [hout, r] blocks (reference layout): output column c is the dot product

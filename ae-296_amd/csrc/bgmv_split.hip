@@ -104,9 +104,9 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
             cv[u] = c < ncc_in;
             const int cs = c < ncc_in ? c : ncc_in - 1;
 #pragma unroll
-            for (int k = 0; k < G; k++) xv[k][u] = xp[k][cs];
+            for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + cs);
 #pragma unroll
-            for (int i = 0; i < RPG; i++) av[i][u] = ap[i][cs];
+            for (int i = 0; i < RPG; i++) av[i][u] = ldg16_stream(ap[i] + cs);
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
@@ -210,10 +210,10 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
         b_rows_of(0, br);
 #pragma unroll
         for (int jj = 0; jj < EB; jj++)
-            bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+            bv[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
 #pragma unroll
         for (int k = 0; k < G; k++)
-            yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
+            yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
     }
 
     // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
             b_rows_of(j0, br);
 #pragma unroll
             for (int jj = 0; jj < EB; jj++)
-                bv[jj] = br[jj] >= 0 ? ldg16(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+                bv[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
         }
 #pragma unroll
         for (int jj = 0; jj < EB; jj++) {
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
     }
 #pragma unroll
     for (int k = 0; k < G; k++)
-        if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
+        if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
 }
 
 template <int DT, int G, int RMAX>

@@ -18,6 +18,11 @@
 
 namespace mlora {
 
+// Activations and outputs pass through once: streaming (nontemporal) accesses.  A and B rows are
+// re-read by every token tile of a segment and stay ordinary cached loads (measured: streaming them
+// too loses what the other three gain).
+
+
 constexpr int TM = 64;       // tokens per tile
 constexpr int TN = 128;      // output columns per expand step
 constexpr int SG_NT = 256;   // 4 wavefronts, 16 tokens each
@@ -214,9 +219,9 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
         const bool ok = c < ncc;                                // K tail: both operands become zero
         const int cs = ok ? c : ncc - 1;
 #pragma unroll
-        for (int q = 0; q < XP; q++) { xr[q] = xp[q][cs]; if (!ok) xr[q] = zero16(); }
+        for (int q = 0; q < XP; q++) { xr[q] = ldg16_stream(xp[q] + cs); if (!ok) xr[q] = zero16(); }
 #pragma unroll
-        for (int q = 0; q < AP; q++) { ar[q] = ap[q][cs]; if (!ok) ar[q] = zero16(); }
+        for (int q = 0; q < AP; q++) { ar[q] = ldg16(ap[q] + cs); if (!ok) ar[q] = zero16(); }
     };
     if (st0 < st1) load_stage(st0);
 #pragma unroll 1
@@ -380,7 +385,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
                 const int pp = lane + 64 * q, t = pp >> 4, c = pp & 15;
                 const int col = col0 + c * 8;
                 const bool ok = wave * 16 + t < ntok && col < col_end;
-                y_nx[q] = ok ? ldg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col) : zero16();
+                y_nx[q] = ok ? ldg16_stream(y + (size_t)(tok0 + wave * 16 + t) * hout + col) : zero16();
             }
         }
         if constexpr (!BT) {
@@ -468,7 +473,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
                 o[2] = fmaf(scale, d0[2], o[2]); o[3] = fmaf(scale, d0[3], o[3]);
                 o[4] = fmaf(scale, d1[0], o[4]); o[5] = fmaf(scale, d1[1], o[5]);
                 o[6] = fmaf(scale, d1[2], o[6]); o[7] = fmaf(scale, d1[3], o[7]);
-                stg16(y + (size_t)(tok0 + wave * 16 + t) * hout + col, pack8<DT>(o));
+                stg16_stream(y + (size_t)(tok0 + wave * 16 + t) * hout + col, pack8<DT>(o));
             }
         }
     }
