@@ -6,7 +6,7 @@
 // while every compute unit is pulling data.  The fused kernel's unit of work is a whole item
 // (an adapter's A and B rows for one projection, hundreds of KiB) and a decode batch has about
 // one item per compute unit, so a unit that gets two items finishes late and the others idle.
-// Here the unit of work is a 1024-column slice of an item (tens of KiB), there are several
+// Here the unit of work is a 2048-column slice of an item (tens of KiB), there are several
 // slices per compute unit and per phase, and no row is fetched by more than one workgroup.
 // The price is the intermediate (T x slices x rank fp32, a few hundred KiB) going through L2.
 //
@@ -18,10 +18,10 @@
 // Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
 #include "mlora_args.hpp"
 #include "mlora_dev.hpp"
+#include <cstdlib>
 
 namespace mlora {
 
-constexpr int SLICE_CHUNKS = 128;                // 16-byte chunks per slice = 1024 columns
 
 struct ItemId { int b, q; };
 
@@ -34,12 +34,14 @@ __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
     return r;
 }
 
-template <int DT, int G, int RMAX>
+template <int DT, int G, int RMAX, int KSC>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
 {
     constexpr int NW = 4;
     constexpr int RPG = RMAX / 4;                               // rank rows per 16-lane row
-    constexpr int U = (RPG + G) <= 12 ? 2 : 1;                  // column steps kept in flight
+    constexpr int STEPS = KSC / 64;             // 16-chunk steps per wavefront
+    constexpr int UW = (RPG + G) <= 12 ? 2 : 1;
+    constexpr int U = UW < STEPS ? UW : STEPS;                  // column steps kept in flight
     __shared__ float s_part[NW][G][RMAX];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     if (adapter < 0) return;
     const int hin = p.hin[proj];
     const int ncc_in = hin >> 3;
-    const int kc0 = ks * SLICE_CHUNKS;
+    const int kc0 = ks * KSC;
     if (kc0 >= ncc_in) return;                                  // this projection has fewer slices
     int r = rec[2];
     r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
@@ -92,15 +94,15 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
 #pragma unroll
         for (int i = 0; i < RPG; i++) acc[k][i] = 0.f;
 
-    // Each wavefront covers 32 chunks of the slice: two steps of 16 chunks per 16-lane row.
+    // Each wavefront covers a quarter of the slice in steps of 16 chunks per 16-lane row.
 #pragma unroll
-    for (int it0 = 0; it0 < 2; it0 += U) {
+    for (int it0 = 0; it0 < STEPS; it0 += U) {
         uint4 xv[G][U];
         uint4 av[RPG][U];
         bool cv[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int c = kc0 + wave * 32 + (it0 + u) * 16 + cl;
+            const int c = kc0 + wave * (STEPS * 16) + (it0 + u) * 16 + cl;
             cv[u] = c < ncc_in;
             const int cs = c < ncc_in ? c : ncc_in - 1;
 #pragma unroll
@@ -142,10 +144,10 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     }
 }
 
-template <int DT, int G, int RMAX>
-__global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
+template <int DT, int G, int RMAX, int KSC, int NTE>
+__global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 {
-    constexpr int NT = 128;                                     // one 16-byte chunk of the slice per thread
+    constexpr int NT = NTE;                                    // one 16-byte chunk of the slice per thread
     constexpr int EB = RMAX < 16 ? RMAX : 16;                   // B rank rows in flight per lane
     __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
 
@@ -160,8 +162,8 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
     ntok = ntok < G ? ntok : G;
     const int hout = p.hout[proj];
     const int ncc_out = hout >> 3;
-    if (cs * SLICE_CHUNKS >= ncc_out) return;                   // this projection has fewer slices
-    const int cc = cs * SLICE_CHUNKS + tid;
+    if (cs * NTE >= ncc_out) return;                   // this projection has fewer slices
+    const int cc = cs * NTE + tid;
     const bool active = cc < ncc_out;
     const int adapter = rec[1];
     int r = rec[2];
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
     }
 
     // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
-    const int n_ks = ((p.hin[proj] >> 3) + SLICE_CHUNKS - 1) / SLICE_CHUNKS;
+    const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
     for (int e = tid; e < G * RMAX; e += NT) {
         const int k = e / RMAX, j = e - k * RMAX;
         float s = 0.f;
@@ -259,34 +261,86 @@ __global__ __launch_bounds__(128) void bgmv_expand_kernel(const BgmvArgs p)
         if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
 }
 
-template <int DT, int G, int RMAX>
+template <int DT, int G, int RMAX, int KSC, int NTE>
 static int launch_pair(const BgmvArgs &a, hipStream_t s)
 {
     const long long n_sh = (long long)a.n_proj * a.ks_max * a.items_cap;
     const long long n_ex = (long long)a.n_proj * a.cs_max * a.items_cap;
     if (n_sh <= 0 || n_ex <= 0) return 0;
     if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
     int rc = (int)hipGetLastError();
     if (rc) return rc;
-    hipLaunchKernelGGL((bgmv_expand_kernel<DT, G, RMAX>), dim3((unsigned)n_ex), dim3(128), 0, s, a);
+    hipLaunchKernelGGL((bgmv_expand_kernel<DT, G, RMAX, KSC, NTE>), dim3((unsigned)n_ex), dim3(NTE), 0, s, a);
     return (int)hipGetLastError();
 }
+
+#ifdef MLORA_TUNE
+// Experiment build: slice sizes chosen at run time from the environment (fp16, groups 2 and 4 only).
+static int env_int(const char *name, int dflt) { const char *v = getenv(name); return v ? atoi(v) : dflt; }
+template <int DT, int G, int RMAX, int KSC>
+static int launch_nte(const BgmvArgs &a, int nte, hipStream_t s)
+{
+    switch (nte) {
+    case 64: return launch_pair<DT, G, RMAX, KSC, 64>(a, s);
+    case 128: return launch_pair<DT, G, RMAX, KSC, 128>(a, s);
+    default: return launch_pair<DT, G, RMAX, KSC, 256>(a, s);
+    }
+}
+template <int DT, int G, int RMAX>
+static int launch_sliced(const BgmvArgs &a, hipStream_t s)
+{
+    if constexpr (DT == DT_F16 && (G == 2 || G == 4)) {
+        int ksc, nte;
+        bgmv_split_slices(RMAX, &ksc, &nte);
+        switch (ksc) {
+        case 64: return launch_nte<DT, G, RMAX, 64>(a, nte, s);
+        case 128: return launch_nte<DT, G, RMAX, 128>(a, nte, s);
+        default: return launch_nte<DT, G, RMAX, 256>(a, nte, s);
+        }
+    } else {
+        return (int)hipErrorInvalidValue;
+    }
+}
+void bgmv_split_slices(int max_rank, int *ksc, int *nte)
+{
+    *ksc = env_int("MLORA_TUNE_KSC", 256);
+    *nte = env_int("MLORA_TUNE_NTE", 256);
+}
+#else
+// Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
+// with rank x slice width, so wider ranks take narrower slices (measured over 64 / 128 / 256 chunks
+// on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
+template <int RMAX> struct Slices;
+template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
+template <> struct Slices<32> { static constexpr int KSC = 128, NTE = 256; };
+template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
+template <int DT, int G, int RMAX>
+static int launch_sliced(const BgmvArgs &a, hipStream_t s)
+{
+    return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE>(a, s);
+}
+void bgmv_split_slices(int max_rank, int *ksc, int *nte)
+{
+    if (max_rank <= 16) { *ksc = Slices<16>::KSC; *nte = Slices<16>::NTE; }
+    else if (max_rank <= 32) { *ksc = Slices<32>::KSC; *nte = Slices<32>::NTE; }
+    else { *ksc = Slices<64>::KSC; *nte = Slices<64>::NTE; }
+}
+#endif
 
 template <int DT, int RMAX>
 static int launch_group(const BgmvArgs &a, int group, hipStream_t s)
 {
     switch (group) {
-    case 1: return launch_pair<DT, 1, RMAX>(a, s);
-    case 2: return launch_pair<DT, 2, RMAX>(a, s);
-    case 4: return launch_pair<DT, 4, RMAX>(a, s);
+    case 1: return launch_sliced<DT, 1, RMAX>(a, s);
+    case 2: return launch_sliced<DT, 2, RMAX>(a, s);
+    case 4: return launch_sliced<DT, 4, RMAX>(a, s);
     case 8:
-        if constexpr (RMAX <= 32) return launch_pair<DT, 8, RMAX>(a, s);
+        if constexpr (RMAX <= 32) return launch_sliced<DT, 8, RMAX>(a, s);
         else return (int)hipErrorInvalidValue;
     default: return (int)hipErrorInvalidValue;
     }
 }
-
 template <int DT>
 static int launch_split_dt(const BgmvArgs &a, int group, int max_rank, hipStream_t s)
 {

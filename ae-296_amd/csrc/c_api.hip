@@ -113,7 +113,9 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
 {
     if (n_proj < 1 || T < 1 || max_hin < 1) return 0;
-    const int64_t ks = (max_hin + 1023) / 1024;
+    int ksc, nte;
+    mlora::bgmv_split_slices(max_rank, &ksc, &nte);
+    const int64_t ks = (max_hin + ksc * 8 - 1) / (ksc * 8);
     return (int64_t)n_proj * T * ks * mlora::bgmv_split_rank_stride(max_rank) * (int64_t)sizeof(float);
 }
 
@@ -171,8 +173,10 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
             return fail(MLORA_ENOSPACE, "workspace holds %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
         if (!aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be 16-byte aligned");
         a.vws = static_cast<float *>(workspace);
-        a.ks_max = (max_hin + 1023) / 1024;
-        a.cs_max = (max_hout + 1023) / 1024;
+        int ksc, nte;
+        mlora::bgmv_split_slices(max_rank, &ksc, &nte);
+        a.ks_max = (max_hin + ksc * 8 - 1) / (ksc * 8);
+        a.cs_max = (max_hout + nte * 8 - 1) / (nte * 8);
         rc = mlora::launch_bgmv_split(a, dtype, group, max_rank, static_cast<hipStream_t>(stream));
     } else {
         rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));

@@ -51,8 +51,8 @@ struct BgmvArgs {
     int n_proj;
     int accumulate;
     float *vws;                    // two-launch form: partial sums [n_proj, T, ks_max, rank stride] (else nullptr)
-    int ks_max;                    // 1024-column slices of the widest hin
-    int cs_max;                    // 1024-column slices of the widest hout
+    int ks_max;                    // shrink slices of the widest hin
+    int cs_max;                    // expand slices of the widest hout
 };
 
 struct GatherArgs {
@@ -103,6 +103,7 @@ struct SgmvArgs {
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);
 int bgmv_split_rank_stride(int max_rank);
+void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);
 constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
 constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)

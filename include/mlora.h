@@ -123,7 +123,7 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T,
  * With work == NULL every token is its own work item and group must be 1.
  * Two-launch form: with a `workspace` of mlora_bgmv_workspace_bytes(n_proj, T, max hin, max_rank)
  * bytes (and work records) the call runs as a shrink launch and an expand launch over
- * 1024-column slices of the items, the fp32 intermediate passing through the workspace; on a
+ * column slices of the items (1024 or 2048 columns, by max_rank), the fp32 intermediate passing through the workspace; on a
  * decode batch with about one item per compute unit this balances the load far better than the
  * fused launch.  workspace == NULL selects the fused launch.  Both forms accumulate in fp32 and
  * round once; they differ only in the order the fp32 partial sums of the shrink are added.

@@ -58,7 +58,7 @@ def test_validation_errors_without_gpu():
     assert bgmv(ws=16, ws_bytes=1 << 20) == _ext.MLORA_EINVAL            # two-launch form without work records
     assert b"work records" in lib.mlora_last_error()
     assert bgmv(ws=16, ws_bytes=64, work=16, group=4) == _ext.MLORA_ENOSPACE
-    assert lib.mlora_bgmv_workspace_bytes(4, 256, 4096, 16) == 4 * 256 * 4 * 16 * 4
+    assert lib.mlora_bgmv_workspace_bytes(4, 256, 4096, 16) == 4 * 256 * 2 * 16 * 4
     assert lib.mlora_bgmv_workspace_bytes(1, 10, 11008, 33) == 10 * 11 * 64 * 4
     assert bgmv(max_pages=1, page_rows=8, max_rank=16) == _ext.MLORA_ERANGE
     assert bgmv(hin=(C.c_int32 * 8)(60, 0, 0, 0, 0, 0, 0, 0)) == _ext.MLORA_EALIGN
