@@ -28,11 +28,11 @@ for _p in (ROOT, os.path.join(ROOT, "ae-296_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per BGMV launch of the default workload, from the two counter runs summarised in
+# HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
 # profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
 # same runs).  Reported as roofline.traffic only when the run is that same configuration.
-MEASURED_TRAFFIC_C2 = 81.28e6
-MEASURED_TRAFFIC_C4_STEP = 3326.5e6
+MEASURED_TRAFFIC_C2 = 81.76e6
+MEASURED_TRAFFIC_C4_STEP = 3249.0e6
 
 
 def log(*a):
@@ -134,15 +134,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
     ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
     ap.add_argument("--fused", action="store_true", help="one fused launch per layer instead of the shrink + expand pair")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c4"],
-                    help="c2 = decode BGMV (the headline metric), c4 = prefill SGMV on Llama-13B shapes")
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+                    help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
+                         "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -169,28 +170,90 @@ def main():
         del src, dst
     if args.workload == "c4":
         return bench_c4(args, dev)
-    L = args.layers
-    log(f"building config 2 with {L} layers ...")
-    wl = workloads.config2(n_layers=L, device=dev)
+    return bench_decode(args, dev)
+
+
+# Decode workloads.  `inputs` names the activation tensor each projection reads (projections that
+# read the same tensor in the model share it here).  `layers` is chosen so that a step's working
+# set is far larger than the 256 MB last-level cache.
+_IN = {"q": "attn", "k": "attn", "v": "attn", "o": "o", "gate": "ffn", "up": "ffn", "down": "down"}
+DECODE = {
+    "c1": dict(desc="config 1: single LoRA-delta op, q_proj 4096->4096, 32 decode tokens, 8 rank-16 adapters, "
+                    "uniform adapter per token, fp16, scaling 2.0",
+               projs=["q"], shapes="7b_attn", T=32, N=8, ranks=[16], alpha=0.0, layers=256, seed=1001),
+    "c2": dict(desc="config 2: decode BGMV, Llama-7B q/k/v/o 4096->4096, 256 tokens, 64 rank-16 adapters, "
+                    "Zipf(1.0), fp16, scaling 2.0",
+               projs=["q", "k", "v", "o"], shapes="7b_attn", T=256, N=64, ranks=[16], alpha=1.0, layers=32, seed=1002),
+    "c3": dict(desc="config 3: heterogeneous-rank decode BGMV, 128 adapters with ranks from {8,16,32,64} in a paged "
+                    "pool, Llama-7B q/k/v/o, gate/up, down, 128 tokens, Zipf(1.2), fp16, scaling 32/r",
+               projs=["q", "k", "v", "o", "gate", "up", "down"], shapes="7b_all", T=128, N=128, ranks=None, alpha=1.2,
+               layers=4, seed=1003),
+    "c5": dict(desc="config 5: one decode step of a Llama-2-7B-shaped LoRA path, 32 layers x 7 projections, 1000 rank-32 "
+                    "adapters resident in a paged pool, 512 decode tokens Zipf(1.1), plus 8 prefill segments of 512 "
+                    "tokens through SGMV in the same step, fp16",
+               projs=["q", "k", "v", "o", "gate", "up", "down"], shapes="7b_all", T=512, N=1000, ranks=[32], alpha=1.1,
+               layers=32, seed=1005, prefill=(8, 512)),
+}
+
+
+def bench_decode(args, dev):
+    import numpy as np
+    import torch
+
+    import mlora
+    from mlora import workloads
+
+    cfg = DECODE[args.workload]
+    L = args.layers if args.layers > 0 else cfg["layers"]
+    shapes = workloads.LLAMA7B_ATTN if cfg["shapes"] == "7b_attn" else workloads.LLAMA7B_ALL
+    projs = cfg["projs"]
+    shapes = {p: shapes[p] for p in projs}
+    rng = np.random.default_rng(cfg["seed"])
+    ranks = cfg["ranks"] if cfg["ranks"] is not None else rng.choice([8, 16, 32, 64], size=cfg["N"]).astype(np.int32)
+    log(f"building {args.workload} with {L} layers ...")
+    wl = workloads.make_decode(args.workload, shapes, L, cfg["T"], cfg["N"], ranks, cfg["alpha"], seed=cfg["seed"],
+                               device=dev, alpha_lora=32.0)
     pool, T = wl.pool, len(wl.tok_adapter)
-    projs = ["q", "k", "v", "o"]
+    log(f"pool slabs: {sum(t.numel() * 2 for t in list(pool.a_rows.values()) + list(pool.b_rows.values())) / 1e9:.2f} GB")
     tok = torch.from_numpy(wl.tok_adapter).to(dev)
     gen = torch.Generator(device=dev)
-    gen.manual_seed(2002)
-    x_qkv = [torch.randn(T, 4096, device=dev, generator=gen).half() for _ in range(L)]
-    x_o = [torch.randn(T, 4096, device=dev, generator=gen).half() for _ in range(L)]
-    ys = [[torch.randn(T, 4096, device=dev, generator=gen).half() for _ in projs] for _ in range(L)]
+    gen.manual_seed(cfg["seed"] + 1000)
+    inputs = sorted({_IN[p] for p in projs})
+    width = {_IN[p]: shapes[p][0] for p in projs}
+    xs = [{i: torch.randn(T, width[i], device=dev, generator=gen).half() for i in inputs} for _ in range(L)]
+    ys = [[torch.randn(T, shapes[p][1], device=dev, generator=gen).half() for p in projs] for _ in range(L)]
     plan = mlora.plan_decode(tok, pool, group=args.group) if args.group else None
     fused = bool(args.fused or plan is None)
 
+    # config 5 carries prefill segments through SGMV in the same step (activations shared by the layers:
+    # they are larger than the last-level cache anyway)
+    pre = None
+    if cfg.get("prefill"):
+        n_seg, seg_len = cfg["prefill"]
+        Tp = n_seg * seg_len
+        seg_adapter = workloads.zipf_adapters(rng, n_seg, cfg["N"], cfg["alpha"])
+        ss = torch.arange(0, Tp, seg_len, dtype=torch.int32, device=dev)
+        sl = torch.full((n_seg,), seg_len, dtype=torch.int32, device=dev)
+        sa = torch.from_numpy(seg_adapter).to(dev)
+        px = {i: torch.randn(Tp, width[i], device=dev, generator=gen).half() for i in inputs}
+        py = {p: torch.randn(Tp, shapes[p][1], device=dev, generator=gen).half() for p in projs}
+        pre = dict(ss=ss, sl=sl, sa=sa, T=Tp, x=px, y=py, ws=mlora.sgmv_workspace(Tp, n_seg, dev), adapters=seg_adapter)
+
     def bgmv_layers():
         for l in range(L):
-            mlora.bgmv(ys[l], [x_qkv[l], x_qkv[l], x_qkv[l], x_o[l]], pool, l, projs, tok, plan=plan, fused=fused)
+            mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
 
     def step():
         if plan is not None:
             mlora.plan_decode(tok, pool, group=args.group, out=plan)
-        bgmv_layers()
+        if pre is None:
+            bgmv_layers()
+            return
+        pplan = mlora.plan_prefill(pre["ss"], pre["sl"], pre["sa"], pre["T"], pool, workspace=pre["ws"])
+        for l in range(L):
+            mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
+            for p in projs:
+                mlora.sgmv(pre["y"][p], pre["x"][_IN[p]], pool, l, p, accumulate=True, plan=pplan)
 
     step()
     torch.cuda.synchronize()
@@ -221,38 +284,49 @@ def main():
     ms = timed(run_step, args.steps)
     wall = time.perf_counter() - t_wall
     ms_per_step = ms / args.steps
-    value = T * len(projs) * L / (ms_per_step * 1e-3)
+    n_tok = T + (pre["T"] if pre else 0)
+    value = n_tok * len(projs) * L / (ms_per_step * 1e-3)
 
-    # The BGMV calls alone: the same 32 layers without the gather, for the roofline figure.
-    run_bgmv = make_runner(bgmv_layers)
-    for _ in range(args.warmup):
-        run_bgmv()
-    ms_k = timed(run_bgmv, args.steps)
-    launch_us = ms_k * 1e3 / (args.steps * L)
     uniq = np.unique(wl.tok_adapter[wl.tok_adapter >= 0])
-    alg = algorithmic_bytes(T, [pool.projections[p] for p in projs], wl.ranks[uniq])
-    achieved = alg / (launch_us * 1e-6) / 1e9
+    shp = [shapes[p] for p in projs]
+    alg = algorithmic_bytes(T, shp, wl.ranks[uniq])
     per_token_gather = sum(T * h[0] * 2 + 2 * T * h[1] * 2 + int(wl.ranks[wl.tok_adapter].sum()) * (h[0] + h[1]) * 2 + 4 * T
-                           for h in (pool.projections[p] for p in projs))
+                           for h in shp)
+    if pre is None:
+        # The BGMV calls alone: the same layers without the gather, for the roofline figure.
+        run_bgmv = make_runner(bgmv_layers)
+        for _ in range(args.warmup):
+            run_bgmv()
+        ms_k = timed(run_bgmv, args.steps)
+        launch_us = ms_k * 1e3 / (args.steps * L)
+        achieved = alg / (launch_us * 1e-6) / 1e9
+        kernel = ("bgmv_kernel" if fused else "bgmv_shrink_kernel + bgmv_expand_kernel (one layer's pair)") + \
+                 f", {len(projs)} projections per call"
+        extra = {"launch_us": launch_us, "algorithmic_bytes_per_launch": alg,
+                 "per_token_gather_bytes_per_launch": per_token_gather}
+    else:
+        # Mixed step: decode and prefill bytes of all layers over the whole step (gather and plan included).
+        pu = np.unique(pre["adapters"])
+        alg_pre = algorithmic_bytes(pre["T"], shp, wl.ranks[pu]) + 12 * len(pre["adapters"]) * len(projs)
+        alg_step = (alg + alg_pre) * L
+        achieved = alg_step / (ms_per_step * 1e-3) / 1e9
+        kernel = "whole step: gather + prefill plan + 32 x (decode pair + 7 x SGMV shrink/reduce/expand)"
+        extra = {"algorithmic_bytes_per_step": alg_step, "decode_bytes_per_layer": alg, "prefill_bytes_per_layer": alg_pre}
+    traffic = MEASURED_TRAFFIC_C2 if (args.workload == "c2" and args.group == 4 and L == 32 and not fused) else None
 
     out = {
         "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",
         "value": value, "unit": "token-projections/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "config 2: decode BGMV, Llama-7B q/k/v/o 4096->4096, 256 tokens, 64 rank-16 adapters, "
-                               "Zipf(1.0), fp16, scaling 2.0",
-                   "layers": L, "projections_per_launch": len(projs), "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0),
+        "config": {"workload": cfg["desc"], "layers": L, "projections_per_call": len(projs),
+                   "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0) + ((1 + 3 * len(projs) * L) if pre else 0),
                    "form": "fused" if fused else "shrink + expand",
-                   "tokens": T, "adapters": 64, "adapters_touched": int(len(uniq)), "group": args.group,
+                   "tokens": T, "prefill_tokens": pre["T"] if pre else 0, "adapters": cfg["N"],
+                   "adapters_touched": int(len(uniq)), "group": args.group,
                    "hip_graph": not args.no_graph, "wall_s_timed_region": wall},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_C2 if (args.group == 4 and L == 32 and not fused) else None,
-                     "kernel": "bgmv_kernel (4 projections per launch)" if fused else
-                               "bgmv_shrink_kernel + bgmv_expand_kernel (one layer's pair, 4 projections)",
-                     "launch_us": launch_us,
-                     "algorithmic_bytes_per_launch": alg, "per_token_gather_bytes_per_launch": per_token_gather},
+        "roofline": dict({"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                          "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": kernel}, **extra),
         "cpu_baseline": None,
     }
     if not args.no_cpu:
