@@ -34,19 +34,101 @@ __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
     return r;
 }
 
-template <int DT, int G, int RMAX, int KSC>
-__global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
+// Shrink of one (item, projection, column slice) over the first 4 * NR rank rows (NR per 16-lane
+// row).  The caller picks the smallest NR that covers the item's rank, so an adapter of rank 8 in a
+// pool that goes up to rank 64 issues loads for 8 rows, not 64.
+template <int DT, int G, int RMAX, int KSC, int NR>
+__device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__restrict__ rows, const int (&tok)[G],
+                                            int r, int proj, int ks, float (&s_part)[4][G][RMAX])
 {
     constexpr int NW = 4;
-    constexpr int RPG = RMAX / 4;                               // rank rows per 16-lane row
-    constexpr int STEPS = KSC / 64;             // 16-chunk steps per wavefront
-    constexpr int UW = (RPG + G) <= 12 ? 2 : 1;
+    constexpr int STEPS = KSC / 64;                             // 16-chunk steps per wavefront
+    constexpr int UW = (NR + G) <= 12 ? 2 : 1;
     constexpr int U = UW < STEPS ? UW : STEPS;                  // column steps kept in flight
-    __shared__ float s_part[NW][G][RMAX];
-
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int cl = lane & 15, rg = lane >> 4;
     const PoolView &pv = p.pool;
+    const int hin = p.hin[proj];
+    const int ncc_in = hin >> 3;
+    const int kc0 = ks * KSC;
+    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x[proj]);
+    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows[proj]);
+
+    // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot beyond
+    // ntok reads token 0 (both discarded below); a chunk past the end of the row re-reads the
+    // last chunk with x forced to zero.
+    const uint4 *ap[NR];
+    unsigned row_ok = 0;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+        int row = rows[rg + 4 * i];
+        row = (row >= 0 && row < pv.n_rows_a) ? row : -1;
+        row_ok |= (row >= 0 ? 1u : 0u) << i;
+        ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+    }
+    const uint4 *xp[G];
+#pragma unroll
+    for (int k = 0; k < G; k++) xp[k] = reinterpret_cast<const uint4 *>(x + (size_t)(tok[k] >= 0 ? tok[k] : 0) * hin);
+    float acc[G][NR];
+#pragma unroll
+    for (int k = 0; k < G; k++)
+#pragma unroll
+        for (int i = 0; i < NR; i++) acc[k][i] = 0.f;
+
+    // Each wavefront covers a quarter of the slice in steps of 16 chunks per 16-lane row.
+#pragma unroll
+    for (int it0 = 0; it0 < STEPS; it0 += U) {
+        uint4 xv[G][U];
+        uint4 av[NR][U];
+        bool cv[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int c = kc0 + wave * (STEPS * 16) + (it0 + u) * 16 + cl;
+            cv[u] = c < ncc_in;
+            const int cs = c < ncc_in ? c : ncc_in - 1;
+#pragma unroll
+            for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + cs);
+#pragma unroll
+            for (int i = 0; i < NR; i++) av[i][u] = ldg16_stream(ap[i] + cs);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int k = 0; k < G; k++) {
+                xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
+                xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
+            }
+#pragma unroll
+            for (int i = 0; i < NR; i++)
+#pragma unroll
+                for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
+        }
+    }
+
+#pragma unroll
+    for (int k = 0; k < G; k++)
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const float a = ((row_ok >> i) & 1u) ? acc[k][i] : 0.f;
+            const float s = row16_sum(a);
+            if (cl == 0) s_part[wave][k][rg + 4 * i] = s;
+        }
+    __syncthreads();
+    for (int e = tid; e < G * 4 * NR; e += 256) {
+        const int k = e / (4 * NR), j = e - k * (4 * NR);
+        if (j < r && tok[k] >= 0) {
+            float s = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; wv++) s += s_part[wv][k][j];
+            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + ks) * RMAX + j] = s;
+        }
+    }
+}
+
+template <int DT, int G, int RMAX, int KSC>
+__global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
+{
+    __shared__ float s_part[4][G][RMAX];
 
     const ItemId id = split_id(blockIdx.x, p.n_proj * p.ks_max);
     const int proj = id.q / p.ks_max, ks = id.q - proj * p.ks_max;
@@ -56,10 +138,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     ntok = ntok < G ? ntok : G;
     const int adapter = rec[1];
     if (adapter < 0) return;
-    const int hin = p.hin[proj];
-    const int ncc_in = hin >> 3;
-    const int kc0 = ks * KSC;
-    if (kc0 >= ncc_in) return;                                  // this projection has fewer slices
+    if (ks * KSC >= (p.hin[proj] >> 3)) return;                 // this projection has fewer slices
     int r = rec[2];
     r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
     int tok[G];
@@ -70,78 +149,15 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     }
     const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
 
-    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x[proj]);
-    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows[proj]);
-
-    // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot beyond
-    // ntok reads token 0 (both discarded below); a chunk past the end of the row re-reads the
-    // last chunk with x forced to zero.
-    const uint4 *ap[RPG];
-    unsigned row_ok = 0;
-#pragma unroll
-    for (int i = 0; i < RPG; i++) {
-        int row = rows[rg + 4 * i];
-        row = (row >= 0 && row < pv.n_rows_a) ? row : -1;
-        row_ok |= (row >= 0 ? 1u : 0u) << i;
-        ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+    // r is uniform over the workgroup: a scalar branch, no divergence.
+    if constexpr (RMAX >= 64) {
+        if (r > 32) { shrink_rows<DT, G, RMAX, KSC, 16>(p, rows, tok, r, proj, ks, s_part); return; }
     }
-    const uint4 *xp[G];
-#pragma unroll
-    for (int k = 0; k < G; k++) xp[k] = reinterpret_cast<const uint4 *>(x + (size_t)(tok[k] >= 0 ? tok[k] : 0) * hin);
-    float acc[G][RPG];
-#pragma unroll
-    for (int k = 0; k < G; k++)
-#pragma unroll
-        for (int i = 0; i < RPG; i++) acc[k][i] = 0.f;
-
-    // Each wavefront covers a quarter of the slice in steps of 16 chunks per 16-lane row.
-#pragma unroll
-    for (int it0 = 0; it0 < STEPS; it0 += U) {
-        uint4 xv[G][U];
-        uint4 av[RPG][U];
-        bool cv[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int c = kc0 + wave * (STEPS * 16) + (it0 + u) * 16 + cl;
-            cv[u] = c < ncc_in;
-            const int cs = c < ncc_in ? c : ncc_in - 1;
-#pragma unroll
-            for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + cs);
-#pragma unroll
-            for (int i = 0; i < RPG; i++) av[i][u] = ldg16_stream(ap[i] + cs);
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-#pragma unroll
-            for (int k = 0; k < G; k++) {
-                xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
-                xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
-            }
-#pragma unroll
-            for (int i = 0; i < RPG; i++)
-#pragma unroll
-                for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
-        }
+    if constexpr (RMAX >= 32) {
+        if (r > 16) { shrink_rows<DT, G, RMAX, KSC, 8>(p, rows, tok, r, proj, ks, s_part); return; }
     }
-
-#pragma unroll
-    for (int k = 0; k < G; k++)
-#pragma unroll
-        for (int i = 0; i < RPG; i++) {
-            const float a = ((row_ok >> i) & 1u) ? acc[k][i] : 0.f;
-            const float s = row16_sum(a);
-            if (cl == 0) s_part[wave][k][rg + 4 * i] = s;
-        }
-    __syncthreads();
-    for (int e = tid; e < G * RMAX; e += 256) {
-        const int k = e / RMAX, j = e - k * RMAX;
-        if (j < r && tok[k] >= 0) {
-            float s = 0.f;
-#pragma unroll
-            for (int wv = 0; wv < NW; wv++) s += s_part[wv][k][j];
-            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + ks) * RMAX + j] = s;
-        }
-    }
+    if (r > 8) { shrink_rows<DT, G, RMAX, KSC, 4>(p, rows, tok, r, proj, ks, s_part); return; }
+    shrink_rows<DT, G, RMAX, KSC, 2>(p, rows, tok, r, proj, ks, s_part);
 }
 
 template <int DT, int G, int RMAX, int KSC, int NTE>
