@@ -57,7 +57,7 @@ class Lora_GPU:
         return w.to(self.dtype).transpose(-1, -2).contiguous()
 
     # ------------------------------------------------------------------ apply
-    def _invoke(self, name, x, layer_id, prefill):
+    def _invoke(self, name, x, layer_id, prefill, lora_ids=None):
         bsz = x.shape[0]
         if prefill:
             down, up = getattr(self, f"{name}_down_prefill"), getattr(self, f"{name}_up_prefill")
@@ -69,19 +69,26 @@ class Lora_GPU:
             if self._workspace is None or self._workspace.numel() < need:
                 self._workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
             return ops.lora_prefill_ref(x, down, up, layer_id, workspace=self._workspace)
-        cur_inds = self.select_inds[bsz - 1]
+        # The reference drops the request's adapter ids (``infer_state.lora_ids``, built at
+        # pre_process.py:50,100) and applies a random stand-in; pass ``lora_ids`` to use the real ones.
+        if lora_ids is None:
+            cur_inds = self.select_inds[bsz - 1]
+        else:
+            if lora_ids.numel() != bsz:
+                raise ValueError("lora_ids must hold one adapter slot per row of x")
+            cur_inds = lora_ids.to(device=x.device, dtype=torch.int64)
         y = torch.zeros(bsz, self.output_size, device=x.device, dtype=x.dtype)
         ops.add_lora_bgmv(y, x, getattr(self, f"{name}_down"), getattr(self, f"{name}_up"), cur_inds, layer_id, 1)
         return y
 
-    def invoke_one_layer_q(self, x, layer_id, prefill=False):
-        return self._invoke("q", x, layer_id, prefill)
+    def invoke_one_layer_q(self, x, layer_id, prefill=False, lora_ids=None):
+        return self._invoke("q", x, layer_id, prefill, lora_ids)
 
-    def invoke_one_layer_k(self, x, layer_id, prefill=False):
-        return self._invoke("k", x, layer_id, prefill)
+    def invoke_one_layer_k(self, x, layer_id, prefill=False, lora_ids=None):
+        return self._invoke("k", x, layer_id, prefill, lora_ids)
 
-    def invoke_one_layer_v(self, x, layer_id, prefill=False):
-        return self._invoke("v", x, layer_id, prefill)
+    def invoke_one_layer_v(self, x, layer_id, prefill=False, lora_ids=None):
+        return self._invoke("v", x, layer_id, prefill, lora_ids)
 
     # ------------------------------------------------------------------ slot management
     def prepare_lora_prefill(self, batch_size):

@@ -28,6 +28,16 @@ def zipf_adapters(rng: np.random.Generator, n_tokens: int, n_adapters: int, alph
     return rng.permutation(n_adapters)[ranks].astype(np.int32)
 
 
+def draw_lora_ids(popularity: np.ndarray, n_requests: int, seed: int = 0) -> np.ndarray:
+    """Adapter id per request the way the reference's load generator draws it
+    (``benchmark/client_maf.py:41-42,53``: ``np.random.seed(0)``, then one
+    ``np.random.choice(total_lora_num, p=lora_popular)`` per request): the i-th value returned is
+    the id of the i-th request that client sends."""
+    popularity = np.asarray(popularity, np.float64)
+    rs = np.random.RandomState(seed)
+    return np.array([rs.choice(len(popularity), p=popularity) for _ in range(n_requests)], np.int32)
+
+
 @dataclass
 class Workload:
     name: str
@@ -58,7 +68,7 @@ def fill_pool(pool: AdapterPool, ranks: np.ndarray, scalings: np.ndarray, rng: n
 
 def make_decode(name: str, projections: Dict[str, Tuple[int, int]], n_layers: int, n_tokens: int,
                 n_adapters: int, ranks, alpha: float, seed: int, dtype=torch.float16, device="cuda",
-                alpha_lora: float = 32.0, page_rows: int = 8) -> Workload:
+                alpha_lora: float = 32.0, page_rows: int = 8, tok_adapter=None) -> Workload:
     rng = np.random.default_rng(seed)
     ranks = np.asarray(ranks, np.int32)
     if ranks.size == 1:
@@ -67,7 +77,7 @@ def make_decode(name: str, projections: Dict[str, Tuple[int, int]], n_layers: in
     pool = AdapterPool(n_layers, projections, n_adapters, n_pages, page_rows=page_rows,
                        max_rank=int(ranks.max()), dtype=dtype, device=device)
     fill_pool(pool, ranks, alpha_lora / ranks.astype(np.float32), rng, seed=seed)
-    tok = zipf_adapters(rng, n_tokens, n_adapters, alpha)
+    tok = zipf_adapters(rng, n_tokens, n_adapters, alpha) if tok_adapter is None else np.asarray(tok_adapter, np.int32)
     return Workload(name, pool, tok, ranks, dict(projections), n_layers)
 
 

@@ -141,9 +141,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512"],
                     help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
-                         "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB)")
+                         "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB); "
+                         "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -194,6 +195,15 @@ DECODE = {
                projs=["q", "k", "v", "o", "gate", "up", "down"], shapes="7b_all", T=512, N=1000, ranks=[32], alpha=1.1,
                layers=32, seed=1005, prefill=(8, 512)),
 }
+# Decode batches whose adapter ids are drawn from the reference's measured adapter-popularity vectors
+# (benchmark/maf_lora_popularity/popularity_{128,256,512}.npy, kept as data under tests/golden/) the way its
+# load generator draws them (benchmark/client_maf.py:41-42,53); q/k/v only, as the reference applies LoRA.
+for _n in (128, 256, 512):
+    DECODE[f"maf{_n}"] = dict(
+        desc=f"decode BGMV, Llama-7B q/k/v 4096->4096, 256 running requests, {_n} rank-16 adapters, adapter per "
+             f"request from the reference's popularity_{_n}.npy, fp16, scaling 2.0",
+        projs=["q", "k", "v"], shapes="7b_attn", T=256, N=_n, ranks=[16], alpha=0.0, layers=32, seed=2000 + _n,
+        popularity=os.path.join(ROOT, "tests", "golden", f"maf_popularity_{_n}.npy"))
 
 
 def bench_decode(args, dev):
@@ -211,8 +221,11 @@ def bench_decode(args, dev):
     rng = np.random.default_rng(cfg["seed"])
     ranks = cfg["ranks"] if cfg["ranks"] is not None else rng.choice([8, 16, 32, 64], size=cfg["N"]).astype(np.int32)
     log(f"building {args.workload} with {L} layers ...")
+    lora_ids = None
+    if cfg.get("popularity"):
+        lora_ids = workloads.draw_lora_ids(np.load(cfg["popularity"], allow_pickle=False), cfg["T"], seed=0)
     wl = workloads.make_decode(args.workload, shapes, L, cfg["T"], cfg["N"], ranks, cfg["alpha"], seed=cfg["seed"],
-                               device=dev, alpha_lora=32.0)
+                               device=dev, alpha_lora=32.0, tok_adapter=lora_ids)
     pool, T = wl.pool, len(wl.tok_adapter)
     log(f"pool slabs: {sum(t.numel() * 2 for t in list(pool.a_rows.values()) + list(pool.b_rows.values())) / 1e9:.2f} GB")
     tok = torch.from_numpy(wl.tok_adapter).to(dev)

@@ -84,6 +84,11 @@ def test_lora_gpu_mirror_calls():
         down, up = getattr(g, f"{name}_down"), getattr(g, f"{name}_up")
         want = torch.stack([x[i].float() @ down[inds[i], 1].float().t() @ up[inds[i], 1].float().t() for i in range(5)])
         assert y.shape == (5, 1024) and torch.allclose(y.float(), want, rtol=RTOL, atol=ATOL)
+    # the request's own adapter slots (infer_state.lora_ids, int32 as pre_process.py:100 builds them)
+    ids = torch.tensor([11, 0, 7, 7, 3], dtype=torch.int32, device="cuda")
+    y = g.invoke_one_layer_q(x, 0, False, lora_ids=ids)
+    want = torch.stack([x[i].float() @ g.q_down[ids[i], 0].float().t() @ g.q_up[ids[i], 0].float().t() for i in range(5)])
+    assert torch.allclose(y.float(), want, rtol=RTOL, atol=ATOL)
     xp = torch.randn(3, 20, 1024, device="cuda", dtype=torch.float16)
     for name in "qkv":
         y = getattr(g, f"invoke_one_layer_{name}")(xp, 0, True)

@@ -1,0 +1,46 @@
+"""Workload generators: the reference's adapter-popularity vectors (data fixtures copied from
+benchmark/maf_lora_popularity/) and the per-request adapter draw of its load generator."""
+import os
+
+import numpy as np
+import pytest
+
+from mlora import workloads
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.mark.parametrize("n", [128, 256, 512])
+def test_popularity_vectors_are_probability_vectors(n):
+    p = np.load(os.path.join(GOLDEN, f"maf_popularity_{n}.npy"), allow_pickle=False)
+    assert p.shape == (n,) and p.dtype == np.float64
+    assert np.all(p > 0) and abs(p.sum() - 1.0) < 1e-12
+    # heavy head: the most popular eighth of the adapters carries about 78 % of the requests
+    assert 0.75 < np.sort(p)[::-1][:n // 8].sum() < 0.82
+
+
+def test_draw_lora_ids_follows_the_clients_stream():
+    """benchmark/client_maf.py:41-42,53: np.random.seed(0) once, then np.random.choice(N, p=pop) per request.
+    The legacy global generator seeded with 0 and drawing one id at a time is that stream."""
+    p = np.load(os.path.join(GOLDEN, "maf_popularity_128.npy"), allow_pickle=False)
+    ids = workloads.draw_lora_ids(p, 300, seed=0)
+    state = np.random.get_state()
+    try:
+        np.random.seed(0)
+        want = [np.random.choice(len(p), p=p) for _ in range(300)]
+    finally:
+        np.random.set_state(state)
+    assert ids.dtype == np.int32 and ids.tolist() == want
+    # and it follows the popularity: empirical frequencies of a long draw agree with p
+    many = workloads.draw_lora_ids(p, 20000, seed=1)
+    freq = np.bincount(many, minlength=len(p)) / len(many)
+    top = np.argsort(p)[::-1][:5]
+    assert np.allclose(freq[top], p[top], atol=0.01)
+
+
+def test_zipf_adapters_range_and_skew():
+    rng = np.random.default_rng(0)
+    a = workloads.zipf_adapters(rng, 5000, 64, 1.0)
+    assert a.dtype == np.int32 and a.min() >= 0 and a.max() < 64
+    counts = np.sort(np.bincount(a, minlength=64))[::-1]
+    assert counts[0] > 4 * counts[16]          # p_1 / p_17 = 17 under Zipf(1.0)
