@@ -110,6 +110,41 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
     return MLORA_OK;
 }
 
+int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab, const int32_t *row_elems,
+                       const int32_t *pages, int n_slot_pages, int rank, int page_rows, int64_t n_pages,
+                       int elt_bytes, void *stream)
+{
+    if (n_jobs < 0 || n_jobs > MLORA_SCATTER_MAX_JOBS) return fail(MLORA_ERANGE, "n_jobs must be in 0..%d (got %d)", MLORA_SCATTER_MAX_JOBS, n_jobs);
+    if (n_jobs == 0) return MLORA_OK;
+    if (!src || !dst_slab || !row_elems || !pages) return fail(MLORA_EINVAL, "NULL argument array");
+    if (rank < 1 || rank > MLORA_MAX_RANK) return fail(MLORA_ERANGE, "rank must be in 1..%d (got %d)", MLORA_MAX_RANK, rank);
+    if (page_rows < 1 || page_rows > 64 || (page_rows & (page_rows - 1))) return fail(MLORA_EINVAL, "page_rows must be a power of two in 1..64 (got %d)", page_rows);
+    if (elt_bytes != 1 && elt_bytes != 2 && elt_bytes != 4) return fail(MLORA_EINVAL, "elt_bytes must be 1, 2 or 4 (got %d)", elt_bytes);
+    if (n_pages <= 0 || n_pages * (int64_t)page_rows > 0x7fffffffLL) return fail(MLORA_ERANGE, "n_pages out of range");
+    const int need = (rank + page_rows - 1) / page_rows;
+    if (n_slot_pages < need) return fail(MLORA_ERANGE, "rank %d needs %d pages, %d given", rank, need, n_slot_pages);
+    mlora::ScatterArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int k = 0; k < 64; k++) a.pages[k] = -1;
+    for (int k = 0; k < need; k++) {
+        if (pages[k] < 0 || pages[k] >= n_pages) return fail(MLORA_ERANGE, "page id %d outside [0, %lld)", pages[k], (long long)n_pages);
+        a.pages[k] = pages[k];
+    }
+    for (int j = 0; j < n_jobs; j++) {
+        if (!src[j] || !dst_slab[j]) return fail(MLORA_EINVAL, "job %d: NULL device pointer", j);
+        const int64_t rb = (int64_t)row_elems[j] * elt_bytes;
+        if (row_elems[j] <= 0 || (rb & 15) || rb > 0x7fffffffLL) return fail(MLORA_EALIGN, "job %d: a row must be a positive multiple of 16 bytes", j);
+        if (!aligned16(src[j]) || !aligned16(dst_slab[j])) return fail(MLORA_EALIGN, "job %d: device pointers must be 16-byte aligned", j);
+        a.src[j] = src[j]; a.dst[j] = dst_slab[j]; a.row_bytes[j] = (int)rb;
+    }
+    a.n_jobs = n_jobs; a.rank = rank; a.n_pages = n_pages;
+    a.page_shift = 0;
+    while ((1 << a.page_shift) < page_rows) a.page_shift++;
+    const int rc = mlora::launch_scatter(a, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "scatter launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
 {
     if (n_proj < 1 || T < 1 || max_hin < 1) return 0;

@@ -55,6 +55,16 @@ struct BgmvArgs {
     int cs_max;                    // expand slices of the widest hout
 };
 
+constexpr int SCATTER_MAX_JOBS = 16;
+struct ScatterArgs {
+    const void *src[SCATTER_MAX_JOBS];   // [rank, row_bytes] contiguous rank rows
+    void *dst[SCATTER_MAX_JOBS];         // rows slab base
+    int row_bytes[SCATTER_MAX_JOBS];     // multiple of 16
+    int pages[64];                       // page id of rank rows [k * page_rows, (k + 1) * page_rows)
+    int n_jobs, rank, page_shift;
+    long long n_pages;
+};
+
 struct GatherArgs {
     const int32_t *tok_adapter;
     const int32_t *page_tbl;
@@ -105,6 +115,7 @@ int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hip
 int bgmv_split_rank_stride(int max_rank);
 void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);
+int launch_scatter(const ScatterArgs &a, hipStream_t s);
 constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
 constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)
 int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s);

@@ -23,6 +23,7 @@ MAX_RANK = 64
 GATHER_MAX_T = 8192
 CNT_NSEG, CNT_NVALID, CNT_NCHUNK, CNT_BAD, CNT_WORDS = 0, 1, 2, 3, 8
 WORK_WORDS = 80
+SCATTER_MAX_JOBS = 16
 
 
 def work_cap(T: int) -> int:
@@ -37,6 +38,7 @@ SIGNATURES = {
     "mlora_version": (_i32, []),
     "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+    "mlora_pool_scatter": (_i32, [_i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i32, _vp]),
     "mlora_bgmv_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
                                 _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),

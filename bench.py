@@ -129,6 +129,78 @@ def bench_c4(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_swap(args, dev):
+    """Adapter swap-in (cold start): one rank-64 adapter for q/k/v of a 32-layer, hidden-4096 model (the shape the
+    reference's swapper is started with, shared_tensor.py:23-30) from pinned host memory onto its pool pages.
+    One step = one whole adapter.  Beside it, the copy pattern of the reference's swapper restated with torch
+    (per layer and tensor a pageable host->device copy and a slice assignment, shared_tensor.py:117-147)."""
+    import torch
+
+    import mlora
+    L, H, r = 32, 4096, 64
+    projections = {p: (H, H) for p in "qkv"}
+    pool = mlora.AdapterPool(L, projections, n_slots=4, n_pages=64, page_rows=8, max_rank=r, dtype=torch.float16, device=dev)
+    loader = mlora.AdapterLoader(pool, layers_per_copy=args.layers if args.layers > 0 else 4, first_layer=8)
+    gen = torch.Generator().manual_seed(3003)
+    w = {p: (torch.randn(L, H, r, generator=gen) * 0.001, torch.randn(L, r, H, generator=gen) * 0.001) for p in "qkv"}
+    host = loader.stage(w, r, 0.5)
+    nbytes = host.nbytes
+
+    def one(slot):
+        t0 = time.perf_counter()
+        ticket = loader.load_async(slot, host)
+        t_issue = time.perf_counter() - t0
+        first = None
+        while not ticket.ready(15):                      # the reference's progress code 2: layers 8..15 are in
+            pass
+        first = time.perf_counter() - t0
+        ticket.wait()
+        return t_issue, first, time.perf_counter() - t0
+
+    for i in range(args.warmup):
+        one(i % 4)
+    res = [one(i % 4) for i in range(args.steps)]
+    torch.cuda.synchronize()
+    issue = sum(r_[0] for r_ in res) / len(res)
+    first = sum(r_[1] for r_ in res) / len(res)
+    total = sum(r_[2] for r_ in res) / len(res)
+
+    # the reference's copy pattern on the same box (torch restatement, not the reference's code)
+    dense = [torch.empty((4, L, r, H), dtype=torch.float16, device=dev) for _ in range(6)]
+    cpu_down = [(0.001 * torch.randn(H, r)).half().t().contiguous() for _ in range(L)]
+    cpu_up = [(0.001 * torch.randn(r, H)).half().t().contiguous() for _ in range(L)]
+
+    def ref_style(j):
+        t0 = time.perf_counter()
+        for k in list(range(8, L)) + list(range(0, 8)):
+            for i in range(3):
+                dense[i][j, k] = cpu_up[k].to(dev).t()
+            for i in range(3, 6):
+                dense[i][j, k] = cpu_down[k].to(dev)
+            if k in (15, 23, 31):
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    ref_style(0)
+    n_ref = max(3, args.steps // 5)
+    ref_t = sum(ref_style(i % 4) for i in range(n_ref)) / n_ref
+
+    gbs = nbytes / total / 1e9
+    out = {"metric": "adapter swap-in throughput (host pinned -> pool pages)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": total * 1e3, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
+           "config": {"workload": "swap-in of one rank-64 adapter, q/k/v, 32 layers, hidden 4096, fp16",
+                      "bytes_per_adapter": nbytes, "layers_per_copy": loader.layers_per_copy,
+                      "ms_until_layers_8_15_ready": first * 1e3, "ms_host_time_to_issue": issue * 1e3},
+           "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
+                        "kernel": "host->device copies (copy engine) + scatter_kernel"},
+           "cpu_baseline": {"value": nbytes / ref_t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                            "sample": f"the swapper's copy pattern (pageable host tensors, one copy and one slice assignment per "
+                                      f"layer and tensor) restated with torch, {n_ref} adapters, {ref_t * 1e3:.2f} ms each"}}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -141,10 +213,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap"],
                     help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
                          "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB); "
-                         "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters")
+                         "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters; "
+                         "swap = adapter swap-in from pinned host memory")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -171,6 +244,8 @@ def main():
         del src, dst
     if args.workload == "c4":
         return bench_c4(args, dev)
+    if args.workload == "swap":
+        return bench_swap(args, dev)
     return bench_decode(args, dev)
 
 

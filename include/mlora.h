@@ -106,6 +106,19 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T,
                       int32_t *counters, int32_t *work, void *stream);
 
 /*
+ * Adapter swap-in, device side: place rank rows that arrived from the host as contiguous blocks on
+ * the pages an adapter owns.  For job j (one (layer, projection, side)): src[j] is [rank, row_elems[j]]
+ * contiguous, dst_slab[j] the rows slab it belongs to; rank row k goes to slab row
+ * pages[k / page_rows] * page_rows + k % page_rows.  `pages` is a HOST array of the slot's page ids.
+ * Replaces the per-layer whole-tensor copies of the reference's swapper (shared_tensor.py:117-147)
+ * and of load_lora_prefill (lora_gpu.py:165-188).  Bit-exact copy; up to MLORA_SCATTER_MAX_JOBS jobs.
+ */
+#define MLORA_SCATTER_MAX_JOBS 16
+int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab, const int32_t *row_elems,
+                       const int32_t *pages, int n_slot_pages, int rank, int page_rows, int64_t n_pages,
+                       int elt_bytes, void *stream);
+
+/*
  * Decode (BGMV): for every token t with adapter a = tok_adapter[t] and every projection p
  *     y_p[t] = (accumulate ? y_p[t] : 0) + scaling[a] * (x_p[t] . A_{p,a}) . B_{p,a}
  * shrink and expand fused in one launch, rank-r intermediate kept on chip in fp32.

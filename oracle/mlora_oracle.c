@@ -19,6 +19,7 @@
  * Pinned functions (see tests/test_oracle_*.py):
  *   orc_f16_to_f32 / orc_f32_to_f16 / orc_bf16_* : exhaustive / randomized vs numpy & torch
  *   orc_pool_gather, orc_build_segments, orc_build_chunks, orc_build_work, orc_sgmv_plan : vs numpy closed forms / enumeration
+ *   orc_pool_scatter          : numpy fancy-index assignment
  *   orc_lora_apply_paged      : brute-force fp64 loops, one-hot, scale 0, library matmul
  *   orc_add_lora_bgmv_ref     : same expression through numpy on the reference layout
  *   orc_prefill_bmm_ref       : numpy matmul pairs (the reference's bmm.bmm)
@@ -142,6 +143,23 @@ int orc_pool_gather(const int32_t *tok_adapter, int T,
         out_scale[t] = scaling[a];
         for (int p = 0; p < max_pages; p++)
             out_row_off[(size_t)t * max_pages + p] = p < np ? page_tbl[(size_t)a * max_pages + p] * page_rows : -1;
+    }
+    return ORC_OK;
+}
+
+/* Adapter swap-in: rank row k of a contiguous block goes to slab row
+ * pages[k / page_rows] * page_rows + k % page_rows (what replaces the per-layer tensor
+ * copies of shared_tensor.py:117-147 / lora_gpu.py:165-188).  Plain byte copy. */
+int orc_pool_scatter(const unsigned char *src, unsigned char *dst_slab, int64_t row_bytes,
+                     const int32_t *pages, int n_slot_pages, int rank, int page_rows, int64_t n_pages)
+{
+    if (rank < 0 || page_rows <= 0 || row_bytes <= 0) return ORC_EINVAL;
+    if ((rank + page_rows - 1) / page_rows > n_slot_pages) return ORC_ERANGE;
+    for (int k = 0; k < rank; k++) {
+        int pg = pages[k / page_rows];
+        if (pg < 0 || pg >= n_pages) return ORC_ERANGE;
+        int64_t row = (int64_t)pg * page_rows + k % page_rows;
+        memcpy(dst_slab + row * row_bytes, src + (int64_t)k * row_bytes, (size_t)row_bytes);
     }
     return ORC_OK;
 }

@@ -90,6 +90,19 @@ def pool_gather(tok_adapter, page_tbl, rank, scaling, page_rows):
     return row_off, out_rank, out_scale
 
 
+def pool_scatter(src, dst_slab, pages, page_rows):
+    """In place: rows of `src` [rank, W] onto the pages `pages` of `dst_slab` [n_pages * page_rows, W]."""
+    src = np.ascontiguousarray(src)
+    assert dst_slab.flags["C_CONTIGUOUS"] and dst_slab.dtype == src.dtype and dst_slab.shape[1] == src.shape[1]
+    pages = np.ascontiguousarray(pages, np.int32)
+    fn = lib().orc_pool_scatter
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int64]
+    rc = fn(_p(src), _p(dst_slab), src.shape[1] * src.itemsize, _p(pages), pages.size, src.shape[0], page_rows,
+            dst_slab.shape[0] // page_rows)
+    _check(rc, "pool_scatter")
+    return dst_slab
+
+
 def build_segments(tok_adapter, n_adapters):
     tok_adapter = np.ascontiguousarray(tok_adapter, np.int32)
     T = tok_adapter.size

@@ -159,3 +159,22 @@ def test_cpu_chunk_plan_matches_reference_formulas(batch, tkn, cap):
     for b, a, n in zip(req, tok0, ntok):
         cover[b, a:a + n] += 1
     assert np.all(cover == 1)
+
+
+def test_pool_scatter_is_a_fancy_index_assignment():
+    rng = np.random.default_rng(77)
+    for rank, page_rows, width in [(16, 8, 64), (5, 8, 24), (64, 8, 40), (9, 4, 16), (1, 1, 8), (33, 16, 72)]:
+        n_pages = 23
+        need = -(-rank // page_rows)
+        pages = rng.permutation(n_pages)[:need + 1].astype(np.int32)       # one spare entry that must not be used
+        src = rng.integers(0, 65536, (rank, width)).astype(np.uint16)
+        slab = rng.integers(0, 65536, (n_pages * page_rows, width)).astype(np.uint16)
+        want = slab.copy()
+        k = np.arange(rank)
+        want[pages[k // page_rows] * page_rows + k % page_rows] = src
+        got = orc.pool_scatter(src, slab.copy(), pages, page_rows)
+        assert np.array_equal(got, want)
+    with pytest.raises(IndexError):
+        orc.pool_scatter(src, slab.copy(), np.array([0, 99], np.int32), 16)          # page id outside the slab
+    with pytest.raises(IndexError):
+        orc.pool_scatter(src, slab.copy(), np.array([0], np.int32), 16)              # too few pages for the rank
