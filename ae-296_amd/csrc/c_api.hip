@@ -279,26 +279,30 @@ namespace {
 
 constexpr int SG_TM = 64;   // tokens per tile, as in sgmv_prefill.hip
 
-struct SgmvWs { int max_tiles; int ksplit; size_t off_rec, off_v, off_hi, off_lo, total; };
+struct SgmvWs { int max_tiles; int ksplit; size_t off_rec, off_proj, per_proj, off_hi, off_lo, total; };
 
-SgmvWs sgmv_layout(int T, int n_seg)
+// Workspace: the plan (tile list, tile records: depends on T and n_seg only), then per projection the
+// K-split partial sums and the hi / lo halves of their sum.
+SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
 {
     SgmvWs w;
     w.max_tiles = T / SG_TM + n_seg + 1;
-    int ks = (768 + w.max_tiles - 1) / w.max_tiles;      // about three shrink workgroups per CU
-    w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : ks);
+    // shrink workgroups: about three per CU for a single projection; a call over several projections
+    // has that many already with fewer splits, and fewer splits mean less partial-sum traffic
+    const long long per_split = (long long)w.max_tiles * n_proj;
+    const long long target = n_proj > 1 ? 2048 : 768;
+    long long ks = (target + per_split - 1) / per_split;
+    w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : (int)ks);
     size_t off = ((size_t)w.max_tiles * 3 + 4) * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
     w.off_rec = off;
     off += (size_t)w.max_tiles * 80 * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
-    w.off_v = off;
-    off += (size_t)w.ksplit * T * MLORA_MAX_RANK * sizeof(float);
-    w.off_hi = off;
-    off += (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
-    w.off_lo = off;
-    off += (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
-    w.total = off;
+    w.off_proj = off;
+    w.off_hi = (size_t)w.ksplit * T * MLORA_MAX_RANK * sizeof(float);
+    w.off_lo = w.off_hi + (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
+    w.per_proj = (w.off_lo + (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t) + 255) & ~(size_t)255;
+    w.total = off + w.per_proj * n_proj;
     return w;
 }
 
@@ -309,10 +313,26 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
     a.tile_seg = ip; a.tile_tok0 = ip + w.max_tiles; a.tile_ntok = ip + 2 * (size_t)w.max_tiles;
     a.n_tiles = ip + 3 * (size_t)w.max_tiles;
     a.tile_rec = reinterpret_cast<int32_t *>(base + w.off_rec);
-    a.v = reinterpret_cast<float *>(base + w.off_v);
-    a.vhi = reinterpret_cast<uint16_t *>(base + w.off_hi);
-    a.vlo = reinterpret_cast<uint16_t *>(base + w.off_lo);
-    a.max_tiles = w.max_tiles; a.ksplit = w.ksplit;
+    a.max_tiles = w.max_tiles;
+    for (int p = 0; p < a.n_proj; p++) {
+        char *pb = base + w.off_proj + w.per_proj * p;
+        a.pr[p].v = reinterpret_cast<float *>(pb);
+        a.pr[p].vhi = reinterpret_cast<uint16_t *>(pb + w.off_hi);
+        a.pr[p].vlo = reinterpret_cast<uint16_t *>(pb + w.off_lo);
+        a.pr[p].ksplit = w.ksplit;
+        // 512 columns per expand workgroup amortise the V operand; fewer when that leaves the chip idle
+        int cols = 512;
+        if (a.n_proj == 1)
+            while (cols > 128 && (long long)w.max_tiles * ((a.pr[p].hout + cols - 1) / cols) < 1024) cols >>= 1;
+        a.pr[p].cols = cols;
+        a.pr[p].ncb = (a.pr[p].hout + cols - 1) / cols;
+    }
+    // shrink groups: consecutive projections that read the same activations
+    a.n_grp = 0;
+    for (int p = 0; p < a.n_proj; p++) {
+        if (p > 0 && a.pr[p].x == a.pr[p - 1].x && a.pr[p].hin == a.pr[p - 1].hin) a.grp_n[a.n_grp - 1]++;
+        else { a.grp_first[a.n_grp] = p; a.grp_n[a.n_grp] = 1; a.n_grp++; }
+    }
 }
 
 }  // namespace
@@ -322,37 +342,52 @@ extern "C" {
 int64_t mlora_sgmv_workspace_bytes(int T, int n_seg)
 {
     if (T <= 0 || n_seg <= 0) return 256;
-    return (int64_t)sgmv_layout(T, n_seg).total;
+    return (int64_t)sgmv_layout(T, n_seg, 1).total;
 }
 
-static int sgmv_common(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
+int64_t mlora_sgmv_multi_workspace_bytes(int T, int n_seg, int n_proj)
+{
+    if (T <= 0 || n_seg <= 0 || n_proj < 1 || n_proj > MLORA_MAX_PROJ) return 256;
+    return (int64_t)sgmv_layout(T, n_seg, n_proj).total;
+}
+
+static int sgmv_common(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+                       const void *const *b_rows, const int32_t *hin, const int32_t *hout, const int32_t *seg_start,
                        const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
-                       const int32_t *rank, const float *scaling, int T, int hin, int hout, int n_adapters,
+                       const int32_t *rank, const float *scaling, int T, int n_adapters,
                        int max_pages, int page_rows, int64_t n_pages, int max_rank, int dtype, int accumulate,
                        void *workspace, int64_t workspace_bytes, int phases, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (T < 0 || n_seg < 0) return fail(MLORA_EINVAL, "T and n_seg must be >= 0 (got %d, %d)", T, n_seg);
+    if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
     if (T == 0 || n_seg == 0) return MLORA_OK;
     if (!seg_start || !seg_len || !seg_adapter) return fail(MLORA_EINVAL, "NULL device pointer");
     mlora::SgmvArgs a;
     memset(&a, 0, sizeof(a));
     int rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
     if (rc) return rc;
+    a.n_proj = n_proj;
     if (phases & mlora::SGMV_APPLY) {
-        if (!y || !x || !a_rows || !b_rows) return fail(MLORA_EINVAL, "NULL device pointer");
-        rc = check_dims(hin, hout);
-        if (rc) return rc;
-        if (!aligned16(y) || !aligned16(x) || !aligned16(a_rows) || !aligned16(b_rows))
-            return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
+        if (!y || !x || !a_rows || !b_rows || !hin || !hout) return fail(MLORA_EINVAL, "per-projection arrays must not be NULL");
+        for (int p = 0; p < n_proj; p++) {
+            if (!y[p] || !x[p] || !a_rows[p] || !b_rows[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
+            rc = check_dims(hin[p], hout[p]);
+            if (rc) return rc;
+            if (!aligned16(y[p]) || !aligned16(x[p]) || !aligned16(a_rows[p]) || !aligned16(b_rows[p]))
+                return fail(MLORA_EALIGN, "projection %d: device pointers must be 16-byte aligned", p);
+            a.pr[p].y = y[p]; a.pr[p].x = x[p]; a.pr[p].a_rows = a_rows[p]; a.pr[p].b_rows = b_rows[p];
+            a.pr[p].hin = hin[p]; a.pr[p].hout = hout[p];
+        }
+    } else {
+        a.pr[0].hin = 8; a.pr[0].hout = 8;
     }
-    const SgmvWs w = sgmv_layout(T, n_seg);
+    const SgmvWs w = sgmv_layout(T, n_seg, n_proj);
     if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
     if (workspace_bytes < (int64_t)w.total)
         return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)w.total);
-    a.y = y; a.x = x; a.a_rows = a_rows; a.b_rows = b_rows;
     a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter; a.n_seg = n_seg;
-    a.T = T; a.hin = hin; a.hout = hout; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0;
+    a.T = T; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0;
     carve(a, workspace, w);
     rc = mlora::launch_sgmv(a, dtype, max_rank, phases, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "sgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -365,8 +400,11 @@ int mlora_sgmv(void *y, const void *x, const void *a_rows, const void *b_rows, c
                int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
                int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    return sgmv_common(y, x, a_rows, b_rows, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T, hin,
-                       hout, n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
+    void *ys[1] = {y};
+    const void *xs[1] = {x}, *as[1] = {a_rows}, *bs[1] = {b_rows};
+    const int32_t hi[1] = {hin}, ho[1] = {hout};
+    return sgmv_common(1, ys, xs, as, bs, hi, ho, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T,
+                       n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
                        workspace_bytes, mlora::SGMV_PLAN | mlora::SGMV_APPLY, stream);
 }
 
@@ -375,9 +413,9 @@ int mlora_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, const int3
                     int max_pages, int page_rows, int64_t n_pages, int max_rank, void *workspace,
                     int64_t workspace_bytes, void *stream)
 {
-    return sgmv_common(nullptr, nullptr, nullptr, nullptr, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank,
-                       scaling, T, 8, 8, n_adapters, max_pages, page_rows, n_pages, max_rank, MLORA_F16, 0, workspace,
-                       workspace_bytes, mlora::SGMV_PLAN, stream);
+    return sgmv_common(1, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, seg_start, seg_len, seg_adapter, n_seg,
+                       page_tbl, rank, scaling, T, n_adapters, max_pages, page_rows, n_pages, max_rank, MLORA_F16, 0,
+                       workspace, workspace_bytes, mlora::SGMV_PLAN, stream);
 }
 
 int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,
@@ -386,8 +424,23 @@ int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b
                        int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
                        int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
 {
-    return sgmv_common(y, x, a_rows, b_rows, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T, hin,
-                       hout, n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
+    void *ys[1] = {y};
+    const void *xs[1] = {x}, *as[1] = {a_rows}, *bs[1] = {b_rows};
+    const int32_t hi[1] = {hin}, ho[1] = {hout};
+    return sgmv_common(1, ys, xs, as, bs, hi, ho, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank, scaling, T,
+                       n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
+                       workspace_bytes, mlora::SGMV_APPLY, stream);
+}
+
+int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+                             const void *const *b_rows, const int32_t *hin, const int32_t *hout,
+                             const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                             const int32_t *page_tbl, const int32_t *rank, const float *scaling, int T,
+                             int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                             int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    return sgmv_common(n_proj, y, x, a_rows, b_rows, hin, hout, seg_start, seg_len, seg_adapter, n_seg, page_tbl, rank,
+                       scaling, T, n_adapters, max_pages, page_rows, n_pages, max_rank, dtype, accumulate, workspace,
                        workspace_bytes, mlora::SGMV_APPLY, stream);
 }
 
@@ -408,7 +461,7 @@ int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void 
         return fail(MLORA_EALIGN, "device pointers must be 16-byte aligned");
     if ((int64_t)B * L * r > 0x7fffffffLL) return fail(MLORA_ERANGE, "pool has more than 2^31-1 rank rows");
     const int T = B * Lpad;
-    const SgmvWs w = sgmv_layout(T, B);
+    const SgmvWs w = sgmv_layout(T, B, 1);
     if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
     if (workspace_bytes < (int64_t)w.total)
         return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)w.total);
@@ -421,10 +474,12 @@ int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void 
     pv.n_rows_a = (long long)(B - 1) * L * r + r;
     pv.b_dense_stride = (long long)L * hout * r;
     pv.n_rows_b = 0;
-    a.y = y; a.x = x;
-    a.a_rows = static_cast<const uint16_t *>(A_T) + (size_t)layer_idx * r * hin;
-    a.b_rows = static_cast<const uint16_t *>(B_T) + (size_t)layer_idx * hout * r;
-    a.n_seg = B; a.T = T; a.hin = hin; a.hout = hout; a.accumulate = 0; a.b_transposed = 1; a.seg_uniform_len = Lpad;
+    a.n_proj = 1;
+    a.pr[0].y = y; a.pr[0].x = x;
+    a.pr[0].a_rows = static_cast<const uint16_t *>(A_T) + (size_t)layer_idx * r * hin;
+    a.pr[0].b_rows = static_cast<const uint16_t *>(B_T) + (size_t)layer_idx * hout * r;
+    a.pr[0].hin = hin; a.pr[0].hout = hout;
+    a.n_seg = B; a.T = T; a.accumulate = 0; a.b_transposed = 1; a.seg_uniform_len = Lpad;
     carve(a, workspace, w);
     rc = mlora::launch_sgmv(a, dtype, r, mlora::SGMV_PLAN | mlora::SGMV_APPLY, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "prefill launch failed: %s", hipGetErrorString((hipError_t)rc));

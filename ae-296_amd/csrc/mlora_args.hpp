@@ -82,17 +82,36 @@ struct GatherArgs {
     int32_t *counters;
 };
 
-struct SgmvArgs {
+// One projection of a prefill call.
+struct SgmvProj {
     void *y;
     const void *x;
     const void *a_rows;
     const void *b_rows;
+    float *v;              // [ksplit, T, MAX_RANK] fp32 partial intermediates
+    uint16_t *vhi;         // [T, MAX_RANK] 16-bit hi part of the summed intermediate
+    uint16_t *vlo;         // [T, MAX_RANK] 16-bit lo part
+    int hin, hout;
+    int ksplit;            // K splits of the shrink
+    int cols, ncb;         // expand: columns per workgroup, column blocks
+};
+
+struct SgmvArgs {
+    SgmvProj pr[MAX_PROJ];
+    int n_proj;
+    // Shrink launch: consecutive projections that read the same x form a group; the workgroups of a
+    // group's members that cover the same tokens and K split run back to back on one XCD, so x comes
+    // from HBM once per group.  grp_end[g] = first workgroup id after group g.
+    int n_grp;
+    int grp_first[MAX_PROJ], grp_n[MAX_PROJ];
+    unsigned grp_end[MAX_PROJ];
+    unsigned ex_end[MAX_PROJ];     // expand launch: first workgroup id after projection p
     PoolView pool;
     const int32_t *seg_start;
     const int32_t *seg_len;
     const int32_t *seg_adapter;
     int n_seg;
-    int T, hin, hout;
+    int T;
     int accumulate;
     int b_transposed;      // B given as [hout, r] blocks (reference layout)
     int seg_uniform_len;   // > 0: segment s covers [s*len, (s+1)*len), adapter s (reference prefill)
@@ -102,11 +121,7 @@ struct SgmvArgs {
     int32_t *tile_ntok;
     int32_t *n_tiles;      // [1]
     int32_t *tile_rec;     // [max_tiles * TILE_WORDS] per-tile records (layout below)
-    float *v;              // [ksplit, T, MAX_RANK] fp32 partial intermediates
-    uint16_t *vhi;         // [T, MAX_RANK] 16-bit hi part of the summed intermediate
-    uint16_t *vlo;         // [T, MAX_RANK] 16-bit lo part
     int max_tiles;
-    int ksplit;
 };
 
 // launchers (defined next to their kernels); return hipError_t as int

@@ -67,6 +67,19 @@ __device__ __forceinline__ bool xcd_remap(int w, int n_second, int &tile, int &s
     tile = run * XRUN + i;
     return true;
 }
+// Shrink form: `second` is (K split, member of the projection group) with the member varying faster and
+// the XCD chosen by the split alone, so the members that read the same x slice follow each other on one XCD.
+__device__ __forceinline__ void xcd_remap_group(int w, int n_split, int n_member, int &tile, int &split, int &member)
+{
+    const int r = w & 7, slot = w >> 3;
+    const int i = slot % XRUN;
+    const int s2 = (slot / XRUN) % (n_split * n_member);
+    const int j = slot / (XRUN * n_split * n_member);
+    split = s2 / n_member;
+    member = s2 - split * n_member;
+    const int run = ((r - split) & 7) + 8 * j;
+    tile = run * XRUN + i;
+}
 __host__ __device__ inline long long xcd_grid(int max_tiles, int n_second)
 {
     const long long runs = (max_tiles + XRUN - 1) / XRUN;
@@ -174,8 +187,12 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
     constexpr int AP = (RMAX * CPR + SG_NT - 1) / SG_NT;   // A loads per thread and stage (1, 2 or 4)
     __shared__ __attribute__((aligned(16))) unsigned char s_x[TM * PITCH];
     __shared__ __attribute__((aligned(16))) unsigned char s_a[RMAX * PITCH];
-    int tile, split;
-    xcd_remap(blockIdx.x, p.ksplit, tile, split);
+    int grp = 0;
+    while (grp + 1 < p.n_grp && blockIdx.x >= p.grp_end[grp]) grp++;
+    int tile, split, member;
+    xcd_remap_group((int)(blockIdx.x - (grp ? p.grp_end[grp - 1] : 0u)), p.pr[p.grp_first[grp]].ksplit, p.grp_n[grp],
+                    tile, split, member);
+    const SgmvProj &pj = p.pr[p.grp_first[grp] + member];
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1];
@@ -186,9 +203,9 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 15, g = lane >> 4;
 
-    const int hin = p.hin;
-    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x);
-    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows);
+    const int hin = pj.hin;
+    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(pj.x);
+    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(pj.a_rows);
     const int lrow = tid >> 4, lchk = tid & 15;                // this thread's row (per pass of 16) and chunk
     const uint4 *xp[XP];
 #pragma unroll
@@ -210,7 +227,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
 
     const int ncc = hin >> 3;                                   // 16-byte chunks per row
     const int nstage = (ncc + CPR - 1) / CPR;
-    const int per = (nstage + p.ksplit - 1) / p.ksplit;
+    const int per = (nstage + pj.ksplit - 1) / pj.ksplit;
     const int st0 = split * per;
     const int st1 = st0 + per < nstage ? st0 + per : nstage;
     uint4 xr[XP], ar[AP];
@@ -246,7 +263,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
         }
     }
     // D[token 4g+i][rank m] per 16x16 block; rank columns that do not exist are stored as zero.
-    float *vout = p.v + ((size_t)split * p.T + tok0 + wave * 16) * VSTRIDE;
+    float *vout = pj.v + ((size_t)split * p.T + tok0 + wave * 16) * VSTRIDE;
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
         const int col = nb * 16 + m;
@@ -281,27 +298,28 @@ template <int DT, int RMAX>
 __global__ __launch_bounds__(256) void sgmv_reduce_kernel(const SgmvArgs p)
 {
     constexpr int CPT = RMAX / 8;     // 8-column groups per token
+    const SgmvProj &pj = p.pr[blockIdx.y];
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)p.T * CPT) return;
     const int t = (int)(idx / CPT), c0 = (int)(idx - (long long)t * CPT) * 8;
     float v[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) v[e] = 0.f;
-    for (int sp = 0; sp < p.ksplit; sp++) {
-        const float4_t *vp = reinterpret_cast<const float4_t *>(p.v + ((size_t)sp * p.T + t) * VSTRIDE + c0);
+    for (int sp = 0; sp < pj.ksplit; sp++) {
+        const float4_t *vp = reinterpret_cast<const float4_t *>(pj.v + ((size_t)sp * p.T + t) * VSTRIDE + c0);
         const float4_t a = vp[0], b = vp[1];
         v[0] += a[0]; v[1] += a[1]; v[2] += a[2]; v[3] += a[3];
         v[4] += b[0]; v[5] += b[1]; v[6] += b[2]; v[7] += b[3];
     }
     uint4 hi, lo;
     split_hi_lo<DT>(v, hi, lo);
-    stg16(p.vhi + (size_t)t * VSTRIDE + c0, hi);
-    stg16(p.vlo + (size_t)t * VSTRIDE + c0, lo);
+    stg16(pj.vhi + (size_t)t * VSTRIDE + c0, hi);
+    stg16(pj.vlo + (size_t)t * VSTRIDE + c0, lo);
 }
 
 // ------------------------------------------------------------------ expand
 template <int DT, int RMAX, bool BT>
-__global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, int cols_per_block, int n_colblk)
+__global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p)
 {
     // One workgroup: 64 tokens (16 per wavefront) x cols_per_block output columns, 128 columns per step.
     // The B tile of a step is parked in LDS row-major and read back column-wise with the transposing LDS
@@ -321,8 +339,12 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     typedef __attribute__((address_space(3))) volatile float lds_vfloat;
     typedef __attribute__((address_space(3))) volatile float4_t lds_vfloat4;
 
+    int proj = 0;
+    while (proj + 1 < p.n_proj && blockIdx.x >= p.ex_end[proj]) proj++;
+    const SgmvProj &pj = p.pr[proj];
+    const int cols_per_block = pj.cols;
     int tile, colblk;
-    xcd_remap(blockIdx.x, n_colblk, tile, colblk);
+    xcd_remap((int)(blockIdx.x - (proj ? p.ex_end[proj - 1] : 0u)), pj.ncb, tile, colblk);
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1], r = rec[2];
@@ -330,8 +352,8 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
     const int tok0 = rec[4];
     const PoolView &pv = p.pool;
     if (ntok <= 0 || tok0 < 0 || tok0 + ntok > p.T) return;
-    const int hout = p.hout;
-    uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y);
+    const int hout = pj.hout;
+    uint16_t *__restrict__ y = static_cast<uint16_t *>(pj.y);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 15, g = lane >> 4;
     const int col_begin = colblk * cols_per_block;
@@ -367,11 +389,11 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p, in
         const int c0 = ks * 32 + 8 * g;
         vhi[ks] = zero16(); vlo[ks] = zero16();
         if (c0 < RMAX) {
-            vhi[ks] = ldg16(p.vhi + ((size_t)(tok0 + trow) * VSTRIDE + c0));
-            vlo[ks] = ldg16(p.vlo + ((size_t)(tok0 + trow) * VSTRIDE + c0));
+            vhi[ks] = ldg16(pj.vhi + ((size_t)(tok0 + trow) * VSTRIDE + c0));
+            vlo[ks] = ldg16(pj.vlo + ((size_t)(tok0 + trow) * VSTRIDE + c0));
         }
     }
-    const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(p.b_rows);
+    const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
     const uint16_t *__restrict__ bt = brows + (BT ? (size_t)adapter * (size_t)pv.b_dense_stride : 0);
     __syncthreads();
 
@@ -489,24 +511,33 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
         if (rc) return rc;
     }
     if (!(phases & SGMV_APPLY)) return 0;
-    hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3((unsigned)xcd_grid(a.max_tiles, a.ksplit)), dim3(SG_NT), 0, s, a);
+    // The caller has filled pr[], the shrink groups, ksplit, cols and ncb; the grid ends are set here.
+    SgmvArgs g = a;
+    unsigned end = 0;
+    for (int q = 0; q < g.n_grp; q++) {
+        end += (unsigned)xcd_grid(g.max_tiles, g.pr[g.grp_first[q]].ksplit * g.grp_n[q]);
+        g.grp_end[q] = end;
+    }
+    const unsigned sgrid = end;
+    end = 0;
+    for (int q = 0; q < g.n_proj; q++) {
+        end += (unsigned)xcd_grid(g.max_tiles, g.pr[q].ncb);
+        g.ex_end[q] = end;
+    }
+    const unsigned egrid = end;
+    hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3(sgrid), dim3(SG_NT), 0, s, g);
     rc = (int)hipGetLastError();
     if (rc) return rc;
     {
-        const long long n = (long long)a.T * (RMAX / 8);
-        hipLaunchKernelGGL((sgmv_reduce_kernel<DT, RMAX>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a);
+        const long long n = (long long)g.T * (RMAX / 8);
+        hipLaunchKernelGGL((sgmv_reduce_kernel<DT, RMAX>), dim3((unsigned)((n + 255) / 256), (unsigned)g.n_proj), dim3(256), 0, s, g);
         rc = (int)hipGetLastError();
         if (rc) return rc;
     }
-    // 512 columns per workgroup amortise the V operand; fewer when that leaves the chip idle
-    int cols = 512;
-    while (cols > TN && (long long)a.max_tiles * ((a.hout + cols - 1) / cols) < 1024) cols >>= 1;
-    const int ncb = (a.hout + cols - 1) / cols;
-    const unsigned egrid = (unsigned)xcd_grid(a.max_tiles, ncb);
-    if (a.b_transposed)
-        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, true>), dim3(egrid), dim3(SG_NT), 0, s, a, cols, ncb);
+    if (g.b_transposed)
+        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, true>), dim3(egrid), dim3(SG_NT), 0, s, g);
     else
-        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, false>), dim3(egrid), dim3(SG_NT), 0, s, a, cols, ncb);
+        hipLaunchKernelGGL((sgmv_expand_kernel<DT, RMAX, false>), dim3(egrid), dim3(SG_NT), 0, s, g);
     return (int)hipGetLastError();
 }
 

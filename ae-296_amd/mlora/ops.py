@@ -184,8 +184,11 @@ def add_lora_bgmv(y: torch.Tensor, x: torch.Tensor, wa_T_all: torch.Tensor, wb_T
 
 
 # ---------------------------------------------------------------------- prefill
-def sgmv_workspace(T: int, n_seg: int, device) -> torch.Tensor:
-    nbytes = _ext.lib().mlora_sgmv_workspace_bytes(T, n_seg)
+def sgmv_workspace(T: int, n_seg: int, device, n_proj: int = 1) -> torch.Tensor:
+    """Workspace for a prefill batch of T tokens in n_seg segments; n_proj > 1 sizes it for
+    ``sgmv_multi`` calls of up to that many projections (it then also serves single ``sgmv`` calls)."""
+    lib = _ext.lib()
+    nbytes = max(lib.mlora_sgmv_workspace_bytes(T, n_seg), lib.mlora_sgmv_multi_workspace_bytes(T, n_seg, n_proj))
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
@@ -212,11 +215,12 @@ def _check_segments(seg_start, seg_len, seg_adapter):
 
 
 def plan_prefill(seg_start: torch.Tensor, seg_len: torch.Tensor, seg_adapter: torch.Tensor, T: int,
-                 pool: AdapterPool, workspace: Optional[torch.Tensor] = None) -> PrefillPlan:
-    """Plan a prefill batch once; the plan serves every projection and layer (``sgmv(..., plan=plan)``)."""
+                 pool: AdapterPool, workspace: Optional[torch.Tensor] = None, n_proj: int = 1) -> PrefillPlan:
+    """Plan a prefill batch once; the plan serves every projection and layer (``sgmv(..., plan=plan)``,
+    ``sgmv_multi(..., plan=plan)`` for up to `n_proj` projections per call)."""
     n_seg = _check_segments(seg_start, seg_len, seg_adapter)
     if workspace is None:
-        workspace = sgmv_workspace(T, n_seg, seg_start.device)
+        workspace = sgmv_workspace(T, n_seg, seg_start.device, n_proj)
     pool.sync()
     rc = _ext.lib().mlora_sgmv_plan(
         seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(), n_seg,
@@ -255,6 +259,36 @@ def sgmv(y: torch.Tensor, x: torch.Tensor, pool: AdapterPool, layer: int, proj: 
         n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling),
         T, hin, hout, pool.n_slots, pool.max_pages, pool.page_rows, pool.n_pages, pool.max_rank,
         pool.dtype_code, int(accumulate), workspace.data_ptr(), workspace.numel(), _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
+def sgmv_multi(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPool, layer: int,
+               projs: Sequence[str], plan: PrefillPlan, accumulate: bool = True) -> None:
+    """Prefill LoRA apply for up to 8 projections of one layer against one plan, three launches in all.
+    Projections listed next to each other with the same x tensor (q, k, v; gate, up) share its reads.
+    The plan's workspace must have been sized for this many projections (``plan_prefill(..., n_proj=)``)."""
+    n = len(projs)
+    if not (len(ys) == len(xs) == n) or not 1 <= n <= _ext.MAX_PROJ:
+        raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y and one x each")
+    _need_cuda(*ys, *xs)
+    _need_contig(*ys, *xs)
+    T = plan.T
+    yv, xv, av, bv, hi, ho = _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
+    for i, p in enumerate(projs):
+        hin, hout = pool.projections[p]
+        if xs[i].dtype != pool.dtype or ys[i].dtype != pool.dtype:
+            raise TypeError(f"x and y must have the pool dtype {pool.dtype}")
+        if tuple(xs[i].shape) != (T, hin) or tuple(ys[i].shape) != (T, hout):
+            raise ValueError(f"projection {p}: expected x [{T}, {hin}] and y [{T}, {hout}]")
+        a_ptr, b_ptr = pool.slab_ptrs(layer, p)
+        yv[i], xv[i], av[i], bv[i], hi[i], ho[i] = ys[i].data_ptr(), xs[i].data_ptr(), a_ptr, b_ptr, hin, hout
+    n_seg = _check_segments(plan.seg_start, plan.seg_len, plan.seg_adapter)
+    pool.sync()
+    rc = _ext.lib().mlora_sgmv_multi_planned(
+        n, yv, xv, av, bv, hi, ho, plan.seg_start.data_ptr(), plan.seg_len.data_ptr(), plan.seg_adapter.data_ptr(),
+        n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling), T, pool.n_slots, pool.max_pages,
+        pool.page_rows, pool.n_pages, pool.max_rank, pool.dtype_code, int(accumulate),
+        plan.workspace.data_ptr(), plan.workspace.numel(), _ext.current_stream_ptr())
     _ext.check(rc)
 
 

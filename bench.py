@@ -92,12 +92,20 @@ def bench_c4(args, dev):
     gen.manual_seed(4004)
     x = {h: torch.randn(T, h, device=dev, generator=gen).bfloat16() for h in (5120, 13824)}
     y = {p: torch.randn(T, projections[p][1], device=dev, generator=gen).bfloat16() for p in projections}
-    ws = mlora.sgmv_workspace(T, 16, dev)
+    # q, k, v read the attention input, gate and up the MLP input; o and down have inputs of their own
+    x_o = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
+    x_ffn = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
+    x_in = {"q": x[5120], "k": x[5120], "v": x[5120], "o": x_o, "gate": x_ffn, "up": x_ffn, "down": x[13824]}
+    ws = mlora.sgmv_workspace(T, 16, dev, n_proj=len(projections))
+    names = list(projections)
 
     def step():
         plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)      # once per batch, shared by the projections
-        for p, (hin, hout) in projections.items():
-            mlora.sgmv(y[p], x[hin], pool, 0, p, accumulate=True, plan=plan)
+        if args.fused:                                                     # one call per projection (3 launches each)
+            for p, (hin, hout) in projections.items():
+                mlora.sgmv(y[p], x[hin], pool, 0, p, accumulate=True, plan=plan)
+        else:                                                              # all seven in one call (3 launches)
+            mlora.sgmv_multi([y[p] for p in names], [x_in[p] for p in names], pool, 0, names, plan)
 
     step()
     torch.cuda.synchronize()
@@ -123,7 +131,8 @@ def bench_c4(args, dev):
            "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
                                   "32 rank-64 adapters, bf16", "tokens": T, "segments": 16},
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                        "traffic": MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)",
+                        "traffic": MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
+                                  "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
                         "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
            "cpu_baseline": None}
     print(json.dumps(out), flush=True)
@@ -208,7 +217,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
     ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
-    ap.add_argument("--fused", action="store_true", help="one fused launch per layer instead of the shrink + expand pair")
+    ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
+                         "instead of one call over the seven")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
@@ -325,7 +335,8 @@ def bench_decode(args, dev):
         sa = torch.from_numpy(seg_adapter).to(dev)
         px = {i: torch.randn(Tp, width[i], device=dev, generator=gen).half() for i in inputs}
         py = {p: torch.randn(Tp, shapes[p][1], device=dev, generator=gen).half() for p in projs}
-        pre = dict(ss=ss, sl=sl, sa=sa, T=Tp, x=px, y=py, ws=mlora.sgmv_workspace(Tp, n_seg, dev), adapters=seg_adapter)
+        pre = dict(ss=ss, sl=sl, sa=sa, T=Tp, x=px, y=py, ws=mlora.sgmv_workspace(Tp, n_seg, dev, n_proj=len(projs)),
+                   adapters=seg_adapter)
 
     def bgmv_layers():
         for l in range(L):
@@ -340,8 +351,7 @@ def bench_decode(args, dev):
         pplan = mlora.plan_prefill(pre["ss"], pre["sl"], pre["sa"], pre["T"], pool, workspace=pre["ws"])
         for l in range(L):
             mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
-            for p in projs:
-                mlora.sgmv(pre["y"][p], pre["x"][_IN[p]], pool, l, p, accumulate=True, plan=pplan)
+            mlora.sgmv_multi([pre["y"][p] for p in projs], [pre["x"][_IN[p]] for p in projs], pool, l, projs, pplan)
 
     step()
     torch.cuda.synchronize()
@@ -398,7 +408,7 @@ def bench_decode(args, dev):
         alg_pre = algorithmic_bytes(pre["T"], shp, wl.ranks[pu]) + 12 * len(pre["adapters"]) * len(projs)
         alg_step = (alg + alg_pre) * L
         achieved = alg_step / (ms_per_step * 1e-3) / 1e9
-        kernel = "whole step: gather + prefill plan + 32 x (decode pair + 7 x SGMV shrink/reduce/expand)"
+        kernel = "whole step: gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"
         extra = {"algorithmic_bytes_per_step": alg_step, "decode_bytes_per_layer": alg, "prefill_bytes_per_layer": alg_pre}
     traffic = MEASURED_TRAFFIC_C2 if (args.workload == "c2" and args.group == 4 and L == 32 and not fused) else None
 
@@ -408,7 +418,7 @@ def bench_decode(args, dev):
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": cfg["desc"], "layers": L, "projections_per_call": len(projs),
-                   "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0) + ((1 + 3 * len(projs) * L) if pre else 0),
+                   "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0) + ((1 + 3 * L) if pre else 0),
                    "form": "fused" if fused else "shrink + expand",
                    "tokens": T, "prefill_tokens": pre["T"] if pre else 0, "adapters": cfg["N"],
                    "adapters_touched": int(len(uniq)), "group": args.group,

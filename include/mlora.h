@@ -210,6 +210,24 @@ int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b
                        int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Several projections of one layer against one plan, in three launches in all (shrink, reduce, expand)
+ * instead of three per projection.  y, x, a_rows, b_rows, hin, hout are HOST arrays of n_proj entries as
+ * in mlora_bgmv_multi.  Consecutive projections that are given the same x pointer (q, k, v; gate, up)
+ * share its reads in the shrink launch: their workgroups for the same tokens run back to back on one
+ * XCD, so x comes from HBM once.  The workspace must hold mlora_sgmv_multi_workspace_bytes(T, n_seg,
+ * n_proj) bytes; a plan written by mlora_sgmv_plan into that workspace is valid for any n_proj.
+ * Replaces the three torch.bmm pairs of lora_gpu.py:127-128,145-146,157-158 for one layer.
+ */
+int64_t mlora_sgmv_multi_workspace_bytes(int T, int n_seg, int n_proj);
+int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x,
+                             const void *const *a_rows, const void *const *b_rows,
+                             const int32_t *hin, const int32_t *hout,
+                             const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                             const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                             int T, int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                             int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * The reference's prefill call on its own layout (lora_gpu.py:125-128): request b uses
  * adapter slot b; x [B, Lpad, hin]; A_T [>=B, L, r, hin]; B_T [>=B, L, hout, r];
  * y [B, Lpad, hout] = (x[b] . A_T[b, layer]^T) . B_T[b, layer]^T   (y is overwritten).

@@ -168,3 +168,67 @@ def test_sgmv_equals_bgmv_at_config4_size():
     sgmv(d2, (2 * x).contiguous(), pool, 0, "p", *(torch.from_numpy(a).cuda() for a in seg), accumulate=False)
     torch.cuda.synchronize()
     assert torch.equal(d2, 2 * d1)
+
+
+def test_sgmv_multi_projection_call():
+    """q, k, v (one x) and o (own x, other widths) in one call of three launches: every projection against the
+    oracle, bit for bit on integer-valued inputs, and no effect on rows outside the segments."""
+    from mlora import sgmv_multi
+    rng = np.random.default_rng(74)
+    ranks = [64, 16, 32, 8, 24]
+    shapes = {"q": (512, 512), "k": (512, 256), "v": (512, 256), "o": (768, 512)}
+    ss = np.array([5, 75, 78, 78, 206], np.int32)
+    sl = np.array([70, 3, 0, 128, 65], np.int32)
+    sa = np.array([2, 0, 1, 3, -1], np.int32)
+    T = 280
+    tok = _tok_of(ss, sl, sa, T)
+    for integer in (False, True):
+        pps = {p: PagedPool(np.random.default_rng(80), ranks, hin, hout, page_rows=8, dtype=FP16, integer=integer)
+               for p, (hin, hout) in shapes.items()}
+        for i, p in enumerate(shapes):                # same page table, different weights per projection
+            r2 = np.random.default_rng(90 + i)
+            if integer:
+                pps[p].a_rows = bits_of(r2.integers(-2, 3, pps[p].a_rows.shape).astype(np.float32), FP16)
+                pps[p].b_rows = bits_of(r2.integers(-2, 3, pps[p].b_rows.shape).astype(np.float32), FP16)
+                pps[p].scaling[:] = [1, 2, 0.5, -1, 4]
+            else:
+                pps[p].a_rows = bits_of((r2.standard_normal(pps[p].a_rows.shape) * 0.02).astype(np.float32), FP16)
+                pps[p].b_rows = bits_of((r2.standard_normal(pps[p].b_rows.shape) * 0.02).astype(np.float32), FP16)
+        pool = upload_pool(pps["q"], projections=shapes)
+        pool.h_scaling[:] = pps["q"].scaling
+        pool._dirty = True
+        for p in shapes:
+            pool.a_rows[p][0].copy_(bits_to_torch(pps[p].a_rows, FP16))
+            pool.b_rows[p][0].copy_(bits_to_torch(pps[p].b_rows, FP16))
+        if integer:
+            mk = lambda h: bits_of((rng.integers(-2, 3, (T, h)) * (rng.random((T, h)) < 0.04)).astype(np.float32), FP16)
+            y0 = {p: bits_of(rng.integers(-8, 9, (T, shapes[p][1])).astype(np.float32), FP16) for p in shapes}
+        else:
+            mk = lambda h: bits_of(rng.standard_normal((T, h)).astype(np.float32), FP16)
+            y0 = {p: bits_of(rng.standard_normal((T, shapes[p][1])).astype(np.float32), FP16) for p in shapes}
+        x_qkv, x_o = mk(512), mk(768)
+        xt_qkv, xt_o = bits_to_torch(x_qkv, FP16, "cuda"), bits_to_torch(x_o, FP16, "cuda")
+        ys = {p: bits_to_torch(y0[p], FP16, "cuda") for p in shapes}
+        d = [torch.from_numpy(a).cuda() for a in (ss, sl, sa)]
+        plan = plan_prefill(d[0], d[1], d[2], T, pool, n_proj=4)
+        say(f"sgmv_multi q,k,v,o integer={integer}")
+        sgmv_multi([ys[p] for p in "qkvo"], [xt_qkv, xt_qkv, xt_qkv, xt_o], pool, 0, list("qkvo"), plan)
+        torch.cuda.synchronize()
+        for p in "qkvo":
+            pps[p].scaling[:] = pps["q"].scaling
+            want = oracle_apply(pps[p], x_o if p == "o" else x_qkv, tok, y0[p])
+            got = torch_to_bits(ys[p])
+            assert np.array_equal(got[tok < 0], y0[p][tok < 0])
+            if integer:
+                assert np.abs(f32_of(want, FP16)).max() < 2048
+                assert np.array_equal(got, want), p
+            else:
+                assert_close_bits(got, want, FP16, f"projection {p}")
+        # the same plan still serves single-projection calls
+        y1 = bits_to_torch(y0["k"], FP16, "cuda")
+        sgmv(y1, xt_qkv, pool, 0, "k", plan=plan)
+        torch.cuda.synchronize()
+        if integer:
+            assert torch.equal(y1, ys["k"])
+        else:
+            assert torch.allclose(y1.float(), ys["k"].float(), rtol=RTOL, atol=ATOL)
