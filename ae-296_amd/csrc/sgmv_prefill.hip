@@ -193,6 +193,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
     xcd_remap_group((int)(blockIdx.x - (grp ? p.grp_end[grp - 1] : 0u)), p.pr[p.grp_first[grp]].ksplit, p.grp_n[grp],
                     tile, split, member);
     const SgmvProj &pj = p.pr[p.grp_first[grp] + member];
+    const bool shared_x = p.grp_n[grp] > 1;
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1];
@@ -236,7 +237,12 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
         const bool ok = c < ncc;                                // K tail: both operands become zero
         const int cs = ok ? c : ncc - 1;
 #pragma unroll
-        for (int q = 0; q < XP; q++) { xr[q] = ldg16_stream(xp[q] + cs); if (!ok) xr[q] = zero16(); }
+        for (int q = 0; q < XP; q++) {
+            // x read by one projection only passes through once (streaming hint); x shared by the members
+            // of a group must stay in L2 for the next member
+            xr[q] = shared_x ? ldg16(xp[q] + cs) : ldg16_stream(xp[q] + cs);
+            if (!ok) xr[q] = zero16();
+        }
 #pragma unroll
         for (int q = 0; q < AP; q++) { ar[q] = ldg16(ap[q] + cs); if (!ok) ar[q] = zero16(); }
     };

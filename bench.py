@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
 # profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
 # same runs).  Reported as roofline.traffic only when the run is that same configuration.
-MEASURED_TRAFFIC_C2 = 81.76e6
-MEASURED_TRAFFIC_C4_STEP = 3249.0e6
+MEASURED_TRAFFIC_C2 = 81.79e6
+MEASURED_TRAFFIC_C4_STEP = 2891.9e6
 
 
 def log(*a):
@@ -131,7 +131,7 @@ def bench_c4(args, dev):
            "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
                                   "32 rank-64 adapters, bf16", "tokens": T, "segments": 16},
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                        "traffic": MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
+                        "traffic": None if args.fused else MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
                                   "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
                         "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
            "cpu_baseline": None}
