@@ -211,3 +211,38 @@ def test_bgmv_full_size_properties():
     torch.cuda.synchronize()
     normal = d1.abs() >= 2.0 ** -13
     assert torch.equal(d2[normal], 2 * d1[normal])
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_bgmv_projections_of_different_widths_in_one_call(fused):
+    """Seven projections with the widths of a (scaled-down) MLP + attention block, ragged against the
+    column slices of the two-launch form: 2056 columns = one slice plus one 16-byte chunk."""
+    rng = np.random.default_rng(45)
+    shapes = {"q": (512, 512), "k": (512, 128), "v": (512, 128), "o": (512, 512),
+              "gate": (512, 2056), "up": (512, 2056), "down": (2056, 512)}
+    T, N = 37, 9
+    ranks = rng.choice([8, 16, 32, 64, 5], N)
+    pps = {p: PagedPool(np.random.default_rng(51), ranks, hin, hout, page_rows=8, dtype=BF16) for p, (hin, hout) in shapes.items()}
+    for i, p in enumerate(shapes):
+        r2 = np.random.default_rng(70 + i)
+        pps[p].a_rows = bits_of((r2.standard_normal(pps[p].a_rows.shape) * 0.02).astype(np.float32), BF16)
+        pps[p].b_rows = bits_of((r2.standard_normal(pps[p].b_rows.shape) * 0.02).astype(np.float32), BF16)
+    pool = upload_pool(pps["q"], projections=shapes)
+    for p in shapes:
+        pool.a_rows[p][0].copy_(bits_to_torch(pps[p].a_rows, BF16))
+        pool.b_rows[p][0].copy_(bits_to_torch(pps[p].b_rows, BF16))
+    tok = rng.integers(-1, N, T).astype(np.int32)
+    xin = {512: bits_of(rng.standard_normal((T, 512)).astype(np.float32), BF16),
+           2056: bits_of(rng.standard_normal((T, 2056)).astype(np.float32), BF16)}
+    y0 = {p: bits_of(rng.standard_normal((T, shapes[p][1])).astype(np.float32), BF16) for p in shapes}
+    t = torch.from_numpy(tok).cuda()
+    xs = {h: bits_to_torch(v, BF16, "cuda") for h, v in xin.items()}
+    ys = {p: bits_to_torch(y0[p], BF16, "cuda") for p in shapes}
+    names = list(shapes)
+    say(f"bgmv 7 projections of different widths fused={fused}")
+    bgmv([ys[p] for p in names], [xs[shapes[p][0]] for p in names], pool, 0, names, t,
+         plan=plan_decode(t, pool, group=2), fused=fused)
+    torch.cuda.synchronize()
+    for p in names:
+        want = oracle_apply(pps[p], xin[shapes[p][0]], tok, y0[p])
+        assert_close_bits(torch_to_bits(ys[p]), want, BF16, f"projection {p}")
