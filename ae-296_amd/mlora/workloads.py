@@ -72,7 +72,7 @@ def make_decode(name: str, projections: Dict[str, Tuple[int, int]], n_layers: in
     rng = np.random.default_rng(seed)
     ranks = np.asarray(ranks, np.int32)
     if ranks.size == 1:
-        ranks = np.full(n_adapters, int(ranks), np.int32)
+        ranks = np.full(n_adapters, int(ranks[0]), np.int32)
     n_pages = int(sum((int(r) + page_rows - 1) // page_rows for r in ranks))
     pool = AdapterPool(n_layers, projections, n_adapters, n_pages, page_rows=page_rows,
                        max_rank=int(ranks.max()), dtype=dtype, device=device)

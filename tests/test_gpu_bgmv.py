@@ -246,3 +246,55 @@ def test_bgmv_projections_of_different_widths_in_one_call(fused):
     for p in names:
         want = oracle_apply(pps[p], xin[shapes[p][0]], tok, y0[p])
         assert_close_bits(torch_to_bits(ys[p]), want, BF16, f"projection {p}")
+
+
+def test_bgmv_config5_one_layer_full_pool():
+    """Config 5 at its real pool size for one layer: 1000 rank-32 adapters (32000 rank rows per slab, 5 GB of
+    slabs), 512 decode tokens Zipf(1.1), all seven Llama-7B projections in one call.  Too large for the
+    CPU oracle in a test, so the check is a plain fp32 evaluation on the device, adapter by adapter, of
+    the rows the pool's own page table names (tolerance as everywhere: rtol 1e-2 / atol 1e-3), for both
+    launch forms, plus agreement of the prefill kernels with the decode kernels on the same tokens."""
+    from mlora import plan_prefill, sgmv_multi, workloads
+    wl = workloads.make_decode("c5-layer", workloads.LLAMA7B_ALL, 1, 512, 1000, [32], 1.1, seed=1005, device="cuda")
+    pool = wl.pool
+    names = list(workloads.LLAMA7B_ALL)
+    T = 512
+    tok = torch.from_numpy(wl.tok_adapter).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    xs = {h: torch.randn(T, h, device="cuda", generator=gen).half() for h in (4096, 11008)}
+    y0 = {p: torch.randn(T, workloads.LLAMA7B_ALL[p][1], device="cuda", generator=gen).half() for p in names}
+    want = {p: y0[p].float().clone() for p in names}
+    for a in np.unique(wl.tok_adapter):
+        idx = torch.from_numpy(np.nonzero(wl.tok_adapter == a)[0]).cuda()
+        rows = pool.rows_of(int(a))
+        for p in names:
+            hin, _ = workloads.LLAMA7B_ALL[p]
+            A = pool.a_rows[p][0][rows].float()                 # [r, hin]
+            B = pool.b_rows[p][0][rows].float()                 # [r, hout]
+            want[p][idx] += float(pool.h_scaling[a]) * ((xs[hin][idx].float() @ A.t()) @ B)
+    plan = plan_decode(tok, pool, group=4)
+    got = {}
+    for fused in (False, True):
+        ys = {p: y0[p].clone() for p in names}
+        say(f"bgmv config-5 layer, 1000 adapters, 7 projections, fused={fused}")
+        bgmv([ys[p] for p in names], [xs[workloads.LLAMA7B_ALL[p][0]] for p in names], pool, 0, names, tok, plan=plan,
+             fused=fused)
+        torch.cuda.synchronize()
+        for p in names:
+            assert torch.allclose(ys[p].float(), want[p], rtol=RTOL, atol=ATOL), (p, fused)
+        got[fused] = ys
+    # the same tokens as a prefill batch: sorted by adapter they form segments
+    order = np.argsort(wl.tok_adapter, kind="stable")
+    sorted_ad = wl.tok_adapter[order]
+    starts = np.flatnonzero(np.r_[True, sorted_ad[1:] != sorted_ad[:-1]]).astype(np.int32)
+    lens = np.diff(np.r_[starts, T]).astype(np.int32)
+    o = torch.from_numpy(order).cuda()
+    pplan = plan_prefill(torch.from_numpy(starts).cuda(), torch.from_numpy(lens).cuda(),
+                         torch.from_numpy(sorted_ad[starts].astype(np.int32)).cuda(), T, pool, n_proj=len(names))
+    ys = {p: y0[p][o].contiguous() for p in names}
+    xo = {h: xs[h][o].contiguous() for h in xs}
+    say("sgmv_multi on the same tokens grouped into segments")
+    sgmv_multi([ys[p] for p in names], [xo[workloads.LLAMA7B_ALL[p][0]] for p in names], pool, 0, names, pplan)
+    torch.cuda.synchronize()
+    for p in names:
+        assert torch.allclose(ys[p].float(), want[p][o], rtol=RTOL, atol=ATOL), p
