@@ -59,15 +59,39 @@ def cpu_baseline(seconds=12.0):
     x = rng.standard_normal((T, H)).astype(np.float16).view(np.uint16)
     req_adapter = rng.integers(0, N, T).astype(np.int32)
     cores = max(1, min(16, os.cpu_count() or 1))
-    orc.cpu_lora_batch(x, down, up, req_adapter, 1, 8, cores)          # warm-up
+    pool = orc.CpuLoraPool(cores)                                       # persistent workers, as the reference's are
+    out_buf = np.empty((T, H), np.uint16)
+    pool.run(x, down, up, req_adapter, 1, 8, out_buf)                  # warm-up
     n, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < seconds:
-        orc.cpu_lora_batch(x, down, up, req_adapter, 1, 8, cores)
+        pool.run(x, down, up, req_adapter, 1, 8, out_buf)
         n += 1
     dt = time.perf_counter() - t0
-    return {"value": T * n / dt, "unit": "token-projections/s", "cores": cores, "kind": "port",
-            "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights), {n} repetitions "
-                      f"in {dt:.1f} s, one task per token over {cores} threads"}
+    pool.close()
+    out = {"value": T * n / dt, "unit": "token-projections/s", "cores": cores, "kind": "port",
+           "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights), {n} repetitions "
+                     f"in {dt:.1f} s, one task per token over {cores} persistent worker threads"}
+    # The same expression through the library the reference's workers call (torch CPU matmul, one thread per
+    # worker as shared_tensor.py:35 / runServerCPULoRA.py:83 pin it): one request per call, a few seconds.
+    import torch
+    prev = torch.get_num_threads()
+    try:
+        torch.set_num_threads(1)
+        xt = torch.from_numpy(x.view(np.float16).copy())
+        dn, upt = torch.from_numpy(down), torch.from_numpy(up)
+        m, t1 = 0, time.perf_counter()
+        while time.perf_counter() - t1 < 3.0:
+            for t in range(T):
+                a = int(req_adapter[t])
+                (xt[t:t + 1].float() @ dn[a] @ upt[a]).half()
+            m += 1
+        d1 = time.perf_counter() - t1
+        out["torch_cpu_one_thread"] = {"value": T * m / d1, "unit": "token-projections/s", "cores": 1,
+                                       "sample": f"x.float() @ down @ up -> half per request with torch on one thread, "
+                                                 f"{m} repetitions in {d1:.1f} s"}
+    finally:
+        torch.set_num_threads(prev)
+    return out
 
 
 def bench_c4(args, dev):

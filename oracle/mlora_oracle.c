@@ -25,6 +25,7 @@
  *   orc_prefill_bmm_ref       : numpy matmul pairs (the reference's bmm.bmm)
  *   orc_cpu_lora_worker       : numpy fp32 matmul of the reference's one-line arithmetic
  *   orc_cpu_chunk_plan        : enumeration of the reference's chunk index arithmetic
+ *   orc_cpu_lora_batch, orc_cpu_pool_run : the worker applied chunk by chunk / each other, bit for bit
  */
 #include <stdint.h>
 #include <stddef.h>
@@ -32,6 +33,9 @@
 #include <stdlib.h>
 #include <math.h>
 #include <pthread.h>
+#ifdef __F16C__
+#include <immintrin.h>
+#endif
 
 #define ORC_OK 0
 #define ORC_EINVAL (-1)
@@ -442,17 +446,40 @@ int orc_prefill_bmm_ref(uint16_t *y, const uint16_t *x, const uint16_t *A_T, con
 /* with fp32 weights down [Hin, r], up [r, Hout] (app.py:38-45).        */
 /* ------------------------------------------------------------------ */
 
+/* fp16 <-> fp32 of whole rows.  With F16C the hardware conversions are used (IEEE, round to nearest
+ * even: the same values as orc_f16_to_f32 / orc_f32_to_f16 for every finite input and infinity). */
+static void orc_row_f16_to_f32(const uint16_t *src, float *dst, int n)
+{
+    int i = 0;
+#ifdef __F16C__
+    for (; i + 8 <= n; i += 8)
+        _mm256_storeu_ps(dst + i, _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(src + i))));
+#endif
+    for (; i < n; i++) dst[i] = orc_f16_to_f32(src[i]);
+}
+
+static void orc_row_f32_to_f16(const float *src, uint16_t *dst, int n)
+{
+    int i = 0;
+#ifdef __F16C__
+    for (; i + 8 <= n; i += 8)
+        _mm_storeu_si128((__m128i *)(dst + i), _mm256_cvtps_ph(_mm256_loadu_ps(src + i), _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC));
+#endif
+    for (; i < n; i++) dst[i] = orc_f32_to_f16(src[i]);
+}
+
 int orc_cpu_lora_worker(const uint16_t *x /* [n_tok, Hin] fp16 */, const float *down, const float *up,
                         uint16_t *out /* [n_tok, Hout] fp16 */, int n_tok, int Hin, int Hout, int r)
 {
     if (n_tok < 0 || r <= 0) return ORC_EINVAL;
-    float *tmp = (float *)malloc(sizeof(float) * (size_t)r);
-    float *row = (float *)malloc(sizeof(float) * (size_t)Hout);
-    if (!tmp || !row) { free(tmp); free(row); return ORC_EINVAL; }
+    float *tmp = (float *)malloc(sizeof(float) * ((size_t)r + (size_t)Hout + (size_t)Hin));
+    if (!tmp) return ORC_EINVAL;
+    float *row = tmp + r, *xf = row + Hout;
     for (int t = 0; t < n_tok; t++) {
+        orc_row_f16_to_f32(x + (size_t)t * Hin, xf, Hin);
         for (int j = 0; j < r; j++) tmp[j] = 0.0f;
         for (int k = 0; k < Hin; k++) {
-            float xv = orc_f16_to_f32(x[(size_t)t * Hin + k]);
+            float xv = xf[k];
             const float *d = down + (size_t)k * r;
             for (int j = 0; j < r; j++) tmp[j] += xv * d[j];
         }
@@ -462,9 +489,9 @@ int orc_cpu_lora_worker(const uint16_t *x /* [n_tok, Hin] fp16 */, const float *
             float tv = tmp[j];
             for (int c = 0; c < Hout; c++) row[c] += tv * u[c];
         }
-        for (int c = 0; c < Hout; c++) out[(size_t)t * Hout + c] = orc_f32_to_f16(row[c]);
+        orc_row_f32_to_f16(row, out + (size_t)t * Hout, Hout);
     }
-    free(tmp); free(row);
+    free(tmp);
     return ORC_OK;
 }
 
@@ -540,4 +567,97 @@ int orc_cpu_lora_batch(const uint16_t *x, const float *down, const float *up, ui
     for (int i = 1; i < n_threads; i++) pthread_join(th[i], NULL);
     free(req);
     return ORC_OK;
+}
+
+/* The same batch on a persistent pool of worker threads (created once, woken per batch through a
+ * mutex and condition variables), which is how the reference runs it: its workers are long-lived
+ * processes pinned to cores (lora_cpu/lora_shm_op/app.py:102-167, runServerCPULoRA.py:83) and its
+ * csrc thread pool is a mutex + condition-variable task queue (csrc/tpool.hpp:38-100).  Thread
+ * creation is therefore not part of a timed batch.  Results are identical to orc_cpu_lora_batch. */
+typedef struct orc_cpu_pool {
+    pthread_mutex_t mu;
+    pthread_cond_t wake, done;
+    pthread_t th[256];
+    int n_threads, generation, pending, stop;
+    orc_cpu_job job;            /* tid / n_threads are filled per worker */
+    int ids[256];
+} orc_cpu_pool;
+
+typedef struct { orc_cpu_pool *pool; int tid; } orc_pool_arg;
+static orc_pool_arg orc_pool_args_storage[4][256];
+static int orc_pool_slots_used = 0;
+
+static void *orc_pool_worker(void *arg)
+{
+    orc_pool_arg *pa = (orc_pool_arg *)arg;
+    orc_cpu_pool *p = pa->pool;
+    int seen = 0;
+    for (;;) {
+        pthread_mutex_lock(&p->mu);
+        while (!p->stop && p->generation == seen) pthread_cond_wait(&p->wake, &p->mu);
+        if (p->stop) { pthread_mutex_unlock(&p->mu); return NULL; }
+        seen = p->generation;
+        orc_cpu_job j = p->job;
+        pthread_mutex_unlock(&p->mu);
+        j.tid = pa->tid; j.n_threads = p->n_threads;
+        orc_cpu_thread(&j);
+        pthread_mutex_lock(&p->mu);
+        if (--p->pending == 0) pthread_cond_signal(&p->done);
+        pthread_mutex_unlock(&p->mu);
+    }
+}
+
+void *orc_cpu_pool_create(int n_threads)
+{
+    if (n_threads <= 0 || n_threads > 256 || orc_pool_slots_used >= 4) return NULL;
+    orc_cpu_pool *p = (orc_cpu_pool *)calloc(1, sizeof(orc_cpu_pool));
+    if (!p) return NULL;
+    pthread_mutex_init(&p->mu, NULL);
+    pthread_cond_init(&p->wake, NULL);
+    pthread_cond_init(&p->done, NULL);
+    p->n_threads = n_threads;
+    orc_pool_arg *args = orc_pool_args_storage[orc_pool_slots_used++];
+    for (int i = 0; i < n_threads; i++) {
+        args[i].pool = p; args[i].tid = i;
+        pthread_create(&p->th[i], NULL, orc_pool_worker, &args[i]);
+    }
+    return p;
+}
+
+int orc_cpu_pool_run(void *pool, const uint16_t *x, const float *down, const float *up, uint16_t *out,
+                     const int32_t *req_adapter, int batch, int tkn_num, int cap, int Hin, int Hout, int r)
+{
+    orc_cpu_pool *p = (orc_cpu_pool *)pool;
+    if (!p) return ORC_EINVAL;
+    int cpr = (tkn_num - 1) / cap + 1;
+    int32_t *req = (int32_t *)malloc(sizeof(int32_t) * 3 * (size_t)batch * cpr);
+    if (!req) return ORC_EINVAL;
+    int32_t *tok0 = req + (size_t)batch * cpr, *ntok = tok0 + (size_t)batch * cpr;
+    int32_t nc = 0;
+    int rc = orc_cpu_chunk_plan(batch, tkn_num, cap, req, tok0, ntok, &nc);
+    if (rc) { free(req); return rc; }
+    pthread_mutex_lock(&p->mu);
+    p->job = (orc_cpu_job){x, down, up, out, req_adapter, req, tok0, ntok, nc, tkn_num, Hin, Hout, r, 0, p->n_threads};
+    p->pending = p->n_threads;
+    p->generation++;
+    pthread_cond_broadcast(&p->wake);
+    while (p->pending > 0) pthread_cond_wait(&p->done, &p->mu);
+    pthread_mutex_unlock(&p->mu);
+    free(req);
+    return ORC_OK;
+}
+
+void orc_cpu_pool_destroy(void *pool)
+{
+    orc_cpu_pool *p = (orc_cpu_pool *)pool;
+    if (!p) return;
+    pthread_mutex_lock(&p->mu);
+    p->stop = 1;
+    pthread_cond_broadcast(&p->wake);
+    pthread_mutex_unlock(&p->mu);
+    for (int i = 0; i < p->n_threads; i++) pthread_join(p->th[i], NULL);
+    pthread_mutex_destroy(&p->mu);
+    pthread_cond_destroy(&p->wake);
+    pthread_cond_destroy(&p->done);
+    free(p);
 }

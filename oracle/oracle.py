@@ -268,3 +268,45 @@ def cpu_lora_batch(x, down, up, req_adapter, tkn_num, cap, n_threads=1):
                                   Hin, Hout, r, n_threads)
     _check(rc, "cpu_lora_batch")
     return out
+
+
+class CpuLoraPool:
+    """Persistent worker threads for ``cpu_lora_batch`` (created once, woken per batch): the way the
+    reference runs its CPU workers, so that thread creation is not part of a timed batch."""
+
+    def __init__(self, n_threads: int):
+        fn = lib().orc_cpu_pool_create
+        fn.restype = C.c_void_p
+        fn.argtypes = [C.c_int]
+        self._h = fn(n_threads)
+        if not self._h:
+            raise ValueError("cannot create a CPU worker pool with that many threads")
+        self.n_threads = n_threads
+
+    def run(self, x, down, up, req_adapter, tkn_num, cap, out=None):
+        x = np.ascontiguousarray(x, np.uint16)
+        down = np.ascontiguousarray(down, np.float32)
+        up = np.ascontiguousarray(up, np.float32)
+        req_adapter = np.ascontiguousarray(req_adapter, np.int32)
+        batch = req_adapter.size
+        _, Hin, r = down.shape
+        Hout = up.shape[2]
+        assert x.shape == (batch * tkn_num, Hin)
+        if out is None:
+            out = np.empty((batch * tkn_num, Hout), np.uint16)
+        fn = lib().orc_cpu_pool_run
+        fn.argtypes = [C.c_void_p] * 6 + [C.c_int] * 6
+        rc = fn(self._h, _p(x), _p(down), _p(up), _p(out), _p(req_adapter), batch, tkn_num, cap, Hin, Hout, r)
+        _check(rc, "cpu_pool_run")
+        return out
+
+    def close(self):
+        if self._h:
+            fn = lib().orc_cpu_pool_destroy
+            fn.argtypes = [C.c_void_p]
+            fn.restype = None
+            fn(self._h)
+            self._h = None
+
+    def __del__(self):
+        self.close()

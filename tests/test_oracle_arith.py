@@ -222,3 +222,20 @@ def test_cpu_batch_is_worker_per_chunk(n_threads):
         a = req_adapter[b]
         want = orc.cpu_lora_worker(x[b * tkn:(b + 1) * tkn], down[a], up[a])
         assert np.array_equal(got[b * tkn:(b + 1) * tkn], want)
+
+
+def test_cpu_pool_equals_batch_over_many_wakeups():
+    """The persistent worker pool gives the same bits as the spawn-per-call form, batch after batch."""
+    rng = np.random.default_rng(38)
+    hin, hout, r, N = 64, 48, 8, 6
+    down = (rng.standard_normal((N, hin, r)) * 0.05).astype(np.float32)
+    up = (rng.standard_normal((N, r, hout)) * 0.05).astype(np.float32)
+    pool = orc.CpuLoraPool(3)
+    try:
+        for batch, tkn, cap in [(3, 20, 8), (1, 1, 8), (7, 5, 2), (4, 16, 16), (2, 9, 4)] * 3:
+            x = rng.standard_normal((batch * tkn, hin)).astype(np.float16).view(np.uint16)
+            req_adapter = rng.integers(0, N, batch).astype(np.int32)
+            assert np.array_equal(pool.run(x, down, up, req_adapter, tkn, cap),
+                                  orc.cpu_lora_batch(x, down, up, req_adapter, tkn, cap, 2))
+    finally:
+        pool.close()
