@@ -240,7 +240,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
-    ap.add_argument("--group", type=int, default=4, help="tokens of one adapter per work item (0 = one token each)")
+    ap.add_argument("--group", type=int, default=-1,
+                    help="tokens of one adapter per work item (0 = no plan, one token each; default: by batch size)")
     ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
                          "instead of one call over the seven")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
@@ -323,6 +324,8 @@ def bench_decode(args, dev):
     from mlora import workloads
 
     cfg = DECODE[args.workload]
+    if args.group < 0:
+        args.group = mlora.ops.default_group(cfg["T"])
     L = args.layers if args.layers > 0 else cfg["layers"]
     shapes = workloads.LLAMA7B_ATTN if cfg["shapes"] == "7b_attn" else workloads.LLAMA7B_ALL
     projs = cfg["projs"]
