@@ -1,0 +1,63 @@
+"""HIP graph replays of the decode and prefill steps give the eager results bit for bit, replay after
+replay, with eager work and synchronisations in between (nothing in the library records a memset node
+or allocates during capture once the plan's buffers exist)."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_common import say, upload_pool
+from helpers import FP16, PagedPool
+from mlora import bgmv, plan_decode, plan_prefill, sgmv_multi
+
+pytestmark = pytest.mark.gpu
+
+
+def test_graph_replays_match_eager():
+    rng = np.random.default_rng(91)
+    ranks = [16, 8, 32, 64, 24, 16]
+    H = 512
+    pp = PagedPool(rng, ranks, H, H, page_rows=8, dtype=FP16)
+    pool = upload_pool(pp, projections={"p": (H, H), "o": (H, H)})
+    pool.a_rows["o"][0].normal_(0, 0.02)
+    pool.b_rows["o"][0].normal_(0, 0.02)
+    T = 97
+    tok = torch.from_numpy(rng.integers(-1, len(ranks), T).astype(np.int32)).cuda()
+    lens = np.array([40, 7, 50], np.int32)
+    ss = torch.from_numpy(np.array([0, 40, 47], np.int32)).cuda()
+    sl = torch.from_numpy(lens).cuda()
+    sa = torch.from_numpy(np.array([3, 0, 5], np.int32)).cuda()
+    x = torch.randn(T, H, device="cuda").half()
+    y_dec = [torch.zeros(T, H, device="cuda").half() for _ in range(2)]
+    y_pre = [torch.zeros(T, H, device="cuda").half() for _ in range(2)]
+    y0 = torch.randn(T, H, device="cuda").half()
+    plan = plan_decode(tok, pool, group=4)
+    pplan = plan_prefill(ss, sl, sa, T, pool, n_proj=2)
+
+    def step():
+        for y in y_dec + y_pre:
+            y.copy_(y0)
+        plan_decode(tok, pool, out=plan)
+        bgmv(y_dec, [x, x], pool, 0, ["p", "o"], tok, plan=plan)
+        plan_prefill(ss, sl, sa, T, pool, workspace=pplan.workspace, n_proj=2)
+        sgmv_multi(y_pre, [x, x], pool, 0, ["p", "o"], pplan)
+
+    say("graph: eager reference step")
+    step()                                        # also allocates the plan's intermediate buffer
+    torch.cuda.synchronize()
+    want = [t.clone() for t in y_dec + y_pre]
+    assert not torch.equal(want[0], y0)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for rep in range(4):
+        # eager work of the program itself between the replays
+        for t in y_dec + y_pre:
+            t.fill_(float(rep))
+        scratch = (torch.randn(1 << 20, device="cuda") * 2).sum()
+        torch.cuda.synchronize()
+        say(f"graph: replay {rep}")
+        g.replay()
+        torch.cuda.synchronize()
+        assert scratch.isfinite()
+        for got, w in zip(y_dec + y_pre, want):
+            assert torch.equal(got, w), rep
