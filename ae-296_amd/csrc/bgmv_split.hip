@@ -18,7 +18,6 @@
 // Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
 #include "mlora_args.hpp"
 #include "mlora_dev.hpp"
-#include <cstdlib>
 
 namespace mlora {
 
@@ -291,39 +290,6 @@ static int launch_pair(const BgmvArgs &a, hipStream_t s)
     return (int)hipGetLastError();
 }
 
-#ifdef MLORA_TUNE
-// Experiment build: slice sizes chosen at run time from the environment (fp16, groups 2 and 4 only).
-static int env_int(const char *name, int dflt) { const char *v = getenv(name); return v ? atoi(v) : dflt; }
-template <int DT, int G, int RMAX, int KSC>
-static int launch_nte(const BgmvArgs &a, int nte, hipStream_t s)
-{
-    switch (nte) {
-    case 64: return launch_pair<DT, G, RMAX, KSC, 64>(a, s);
-    case 128: return launch_pair<DT, G, RMAX, KSC, 128>(a, s);
-    default: return launch_pair<DT, G, RMAX, KSC, 256>(a, s);
-    }
-}
-template <int DT, int G, int RMAX>
-static int launch_sliced(const BgmvArgs &a, hipStream_t s)
-{
-    if constexpr (DT == DT_F16 && (G == 2 || G == 4)) {
-        int ksc, nte;
-        bgmv_split_slices(RMAX, &ksc, &nte);
-        switch (ksc) {
-        case 64: return launch_nte<DT, G, RMAX, 64>(a, nte, s);
-        case 128: return launch_nte<DT, G, RMAX, 128>(a, nte, s);
-        default: return launch_nte<DT, G, RMAX, 256>(a, nte, s);
-        }
-    } else {
-        return (int)hipErrorInvalidValue;
-    }
-}
-void bgmv_split_slices(int max_rank, int *ksc, int *nte)
-{
-    *ksc = env_int("MLORA_TUNE_KSC", 256);
-    *nte = env_int("MLORA_TUNE_NTE", 256);
-}
-#else
 // Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
 // with rank x slice width, so wider ranks take narrower slices (measured over 64 / 128 / 256 chunks
 // on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
@@ -342,7 +308,6 @@ void bgmv_split_slices(int max_rank, int *ksc, int *nte)
     else if (max_rank <= 32) { *ksc = Slices<32>::KSC; *nte = Slices<32>::NTE; }
     else { *ksc = Slices<64>::KSC; *nte = Slices<64>::NTE; }
 }
-#endif
 
 template <int DT, int RMAX>
 static int launch_group(const BgmvArgs &a, int group, hipStream_t s)
