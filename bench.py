@@ -31,8 +31,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
 # profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
 # same runs).  Reported as roofline.traffic only when the run is that same configuration.
-MEASURED_TRAFFIC_C2 = 81.79e6
-MEASURED_TRAFFIC_C4_STEP = 2891.9e6
+MEASURED_TRAFFIC_C2 = 81.82e6
+MEASURED_TRAFFIC_C4_STEP = 2887.4e6
 
 
 def log(*a):
