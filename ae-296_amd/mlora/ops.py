@@ -122,7 +122,8 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     (``fused=False``, the default) or as one fused launch (``fused=True``); without a plan it is
     always the fused launch with one token per work item.  The two-launch form keeps its fp32
     intermediate in a buffer owned by the plan, allocated on the first call that needs it (so
-    run one call before capturing a HIP graph)."""
+    run one call before capturing a HIP graph); calls that share a plan must therefore follow each
+    other on one stream, not overlap on several."""
     n = len(projs)
     if not (len(ys) == len(xs) == n) or not 1 <= n <= _ext.MAX_PROJ:
         raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y and one x each")

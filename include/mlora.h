@@ -138,7 +138,8 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
  * bytes (and work records) the call runs as a shrink launch and an expand launch over
  * column slices of the items (1024 or 2048 columns, by max_rank), the fp32 intermediate passing through the workspace; on a
  * decode batch with about one item per compute unit this balances the load far better than the
- * fused launch.  workspace == NULL selects the fused launch.  Both forms accumulate in fp32 and
+ * fused launch.  workspace == NULL selects the fused launch.  Calls that share a workspace must be
+ * ordered on one stream.  Both forms accumulate in fp32 and
  * round once; they differ only in the order the fp32 partial sums of the shrink are added.
  */
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank);
