@@ -145,6 +145,85 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
     return MLORA_OK;
 }
 
+int mlora_host_alloc(int64_t bytes, void **host_ptr, void **dev_ptr)
+{
+    if (bytes <= 0 || !host_ptr || !dev_ptr) return fail(MLORA_EINVAL, "bytes must be positive and the out pointers non-NULL");
+    void *h = nullptr, *d = nullptr;
+    hipError_t e = hipHostMalloc(&h, (size_t)bytes, hipHostMallocMapped | hipHostMallocPortable);
+    if (e != hipSuccess) return fail(MLORA_ELAUNCH, "hipHostMalloc of %lld bytes failed: %s", (long long)bytes, hipGetErrorString(e));
+    e = hipHostGetDevicePointer(&d, h, 0);
+    if (e != hipSuccess) { (void)hipHostFree(h); return fail(MLORA_ELAUNCH, "hipHostGetDevicePointer failed: %s", hipGetErrorString(e)); }
+    memset(h, 0, (size_t)bytes);
+    *host_ptr = h; *dev_ptr = d;
+    return MLORA_OK;
+}
+
+int mlora_host_free(void *host_ptr)
+{
+    if (!host_ptr) return MLORA_OK;
+    const hipError_t e = hipHostFree(host_ptr);
+    if (e != hipSuccess) return fail(MLORA_ELAUNCH, "hipHostFree failed: %s", hipGetErrorString(e));
+    return MLORA_OK;
+}
+
+static int assist_dims(int B, int tkn, int H, int n_slots, int slot_tokens)
+{
+    if (B < 0 || tkn < 0) return fail(MLORA_EINVAL, "B and tkn must be >= 0 (got %d, %d)", B, tkn);
+    if (H <= 0 || (H & 7)) return fail(MLORA_EALIGN, "H must be a positive multiple of 8 (got %d)", H);
+    if (n_slots <= 0 || slot_tokens <= 0) return fail(MLORA_EINVAL, "n_slots and slot_tokens must be positive");
+    if (B > n_slots) return fail(MLORA_ERANGE, "%d requests do not fit %d request slots", B, n_slots);
+    if (tkn > slot_tokens) return fail(MLORA_ERANGE, "%d tokens per request do not fit a slot of %d", tkn, slot_tokens);
+    return MLORA_OK;
+}
+
+int mlora_assist_export(const void *hidden, int B, int tkn, int H, void *x_slots, int n_slots, int slot_tokens,
+                        int16_t *signals, int n_proj, int n_workers, int cap, int sig_base, int sig_stride, void *stream)
+{
+    int rc = assist_dims(B, tkn, H, n_slots, slot_tokens);
+    if (rc) return rc;
+    if (B == 0 || tkn == 0) return MLORA_OK;
+    if (!hidden || !x_slots || !signals) return fail(MLORA_EINVAL, "NULL pointer");
+    if (!aligned16(hidden) || !aligned16(x_slots)) return fail(MLORA_EALIGN, "hidden and x_slots must be 16-byte aligned");
+    if (n_proj < 1 || n_proj > mlora::ASSIST_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", mlora::ASSIST_MAX_PROJ, n_proj);
+    if (cap <= 0) return fail(MLORA_EINVAL, "cap (tokens per worker) must be positive");
+    const int64_t active = (int64_t)B * ((tkn - 1) / cap + 1);      // one worker per (request, chunk of <= cap tokens)
+    if (active > n_workers) return fail(MLORA_ERANGE, "%lld workers needed per projection, %d available", (long long)active, n_workers);
+    if (sig_base < 2 || sig_stride < active || (int64_t)sig_base + (int64_t)sig_stride * n_proj > 32767)
+        return fail(MLORA_ERANGE, "signal codes must be > 1, distinct per projection and fit 16 bits");
+    mlora::AssistArgs a;
+    memset(&a, 0, sizeof(a));
+    a.dev = hidden; a.host_slots[0] = x_slots; a.signals = signals;
+    a.B = B; a.tkn = tkn; a.H = H; a.n_slots = n_slots; a.slot_tokens = slot_tokens;
+    a.n_proj = n_proj; a.n_workers = n_workers; a.n_active = (int)active; a.sig_base = sig_base; a.sig_stride = sig_stride;
+    rc = mlora::launch_assist_export(a, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "export launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+int mlora_assist_import(int n_proj, void *const *res, const void *const *out_slots, int B, int tkn, int H, int out_size,
+                        int col0, int n_slots, int slot_tokens, void *stream)
+{
+    int rc = assist_dims(B, tkn, H, n_slots, slot_tokens);
+    if (rc) return rc;
+    if (B == 0 || tkn == 0) return MLORA_OK;
+    if (n_proj < 1 || n_proj > mlora::ASSIST_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", mlora::ASSIST_MAX_PROJ, n_proj);
+    if (!res || !out_slots) return fail(MLORA_EINVAL, "NULL argument array");
+    if (out_size <= 0 || (out_size & 7) || col0 < 0 || (col0 & 7) || col0 + out_size > H)
+        return fail(MLORA_EALIGN, "out_size and col0 must be multiples of 8 with col0 + out_size <= H");
+    mlora::AssistArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int q = 0; q < n_proj; q++) {
+        if (!res[q] || !out_slots[q]) return fail(MLORA_EINVAL, "projection %d: NULL pointer", q);
+        if (!aligned16(res[q]) || !aligned16(out_slots[q])) return fail(MLORA_EALIGN, "projection %d: pointers must be 16-byte aligned", q);
+        a.dev_out[q] = res[q]; a.host_slots[q] = const_cast<void *>(out_slots[q]);
+    }
+    a.B = B; a.tkn = tkn; a.H = H; a.out = out_size; a.col0 = col0; a.n_slots = n_slots; a.slot_tokens = slot_tokens;
+    a.n_proj = n_proj;
+    rc = mlora::launch_assist_import(a, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "import launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
 {
     if (n_proj < 1 || T < 1 || max_hin < 1) return 0;

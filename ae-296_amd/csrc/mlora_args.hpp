@@ -65,6 +65,18 @@ struct ScatterArgs {
     long long n_pages;
 };
 
+constexpr int ASSIST_MAX_PROJ = 4;
+struct AssistArgs {
+    const void *dev;                       // export: hidden states [B * tkn, H] (device)
+    void *host_slots[ASSIST_MAX_PROJ];     // export: [0] = request slots; import: result slots per projection (mapped host)
+    void *dev_out[ASSIST_MAX_PROJ];        // import: [B, tkn, out] per projection (device)
+    int16_t *signals;                      // [n_proj, n_workers] (mapped host)
+    int B, tkn, H, out, col0;
+    int n_slots, slot_tokens;
+    int n_proj, n_workers, n_active;
+    int sig_base, sig_stride;
+};
+
 struct GatherArgs {
     const int32_t *tok_adapter;
     const int32_t *page_tbl;
@@ -131,6 +143,8 @@ int bgmv_split_rank_stride(int max_rank);
 void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);
 int launch_scatter(const ScatterArgs &a, hipStream_t s);
+int launch_assist_export(const AssistArgs &a, hipStream_t s);
+int launch_assist_import(const AssistArgs &a, hipStream_t s);
 constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
 constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)
 int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s);

@@ -39,6 +39,10 @@ SIGNATURES = {
     "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
     "mlora_pool_scatter": (_i32, [_i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i32, _vp]),
+    "mlora_host_alloc": (_i32, [_i64, _vp, _vp]),
+    "mlora_host_free": (_i32, [_vp]),
+    "mlora_assist_export": (_i32, [_vp, _i32, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
+    "mlora_assist_import": (_i32, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     "mlora_bgmv_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
                                 _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),

@@ -234,6 +234,75 @@ def bench_swap(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_assist(args, dev):
+    """CPU-assist transport alone (no worker arithmetic): hidden states of a prefill batch to the host request
+    slots plus the wake-up codes, and the q/k/v result slots back to the device.  Shape of the reference's
+    CPU-assisted prefill: hidden 4096, slots of 256 tokens, 64 tokens per worker; 8 requests of 256 tokens.
+    Beside it, the reference's call pattern restated with torch (one device->host copy per request, one
+    host->device copy per finished chunk and projection, lora_cpu.py:176-232)."""
+    import torch
+
+    import mlora
+    B, tkn, H, cap = 8, 256, 4096, 64
+    cfg = dict(batch_size=B, lora_num=64, tp_degree=1, hidden_dim=H, lora_rank=16, token_per_lora=cap, n_layers=32)
+    cpu = mlora.Lora_CPU(cfg, gpu_id=0, device=dev)
+    hidden = torch.randn(B * tkn, H, device=dev).half()
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    t_exp = t_imp = 0.0
+    for i in range(args.warmup + args.steps):
+        e[0].record()
+        cpu.invoke_lora_async(hidden, tkn)
+        e[1].record()
+        torch.cuda.synchronize()
+        cpu.np_signal[:] = 0                                   # the workers' part: nothing computed here
+        e[2].record()
+        cpu.collect_qkv(tkn, B)
+        e[3].record()
+        torch.cuda.synchronize()
+        if i >= args.warmup:
+            t_exp += e[0].elapsed_time(e[1])
+            t_imp += e[2].elapsed_time(e[3])
+    t_exp, t_imp = t_exp / args.steps, t_imp / args.steps
+    b_exp, b_imp = B * tkn * H * 2, 3 * B * tkn * H * 2
+
+    # reference call pattern, restated: pinned host tensors, one copy per request out, one per chunk back
+    slots = torch.empty((64, 256, H), dtype=torch.float16, pin_memory=True)
+    outs = [torch.empty((64, 256, H), dtype=torch.float16, pin_memory=True) for _ in range(3)]
+    res = [torch.empty((B, tkn, H), dtype=torch.float16, device=dev) for _ in range(3)]
+    hv = hidden.view(B, tkn, H)
+    cpr = (tkn - 1) // cap + 1
+
+    def ref_style():
+        t0 = time.perf_counter()
+        for b in range(B):
+            slots[b, :tkn].copy_(hv[b], non_blocking=True)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for q in range(3):
+            for b in range(B):
+                for o in range(cpr):
+                    res[q][b, o * cap:(o + 1) * cap].copy_(outs[q][b, o * cap:(o + 1) * cap])      # synchronous, as cudaHtoD2D is
+        torch.cuda.synchronize()
+        return t1 - t0, time.perf_counter() - t1
+
+    ref_style()
+    rr = [ref_style() for _ in range(max(3, args.steps // 5))]
+    r_exp, r_imp = sum(x[0] for x in rr) / len(rr) * 1e3, sum(x[1] for x in rr) / len(rr) * 1e3
+    cpu.close()
+    gbs = (b_exp + b_imp) / ((t_exp + t_imp) * 1e-3) / 1e9
+    out = {"metric": "CPU-assist transport throughput (device <-> pinned host slots)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": t_exp + t_imp, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
+           "config": {"workload": "8 requests x 256 tokens, hidden 4096: export 16.8 MB + wake-up codes, import q/k/v 50.3 MB",
+                      "export_ms": t_exp, "import_ms": t_imp, "export_GBs": b_exp / t_exp / 1e6, "import_GBs": b_imp / t_imp / 1e6},
+           "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
+                        "kernel": "assist_export_kernel + assist_signal_kernel, assist_import_kernel"},
+           "cpu_baseline": {"value": (b_exp + b_imp) / ((r_exp + r_imp) * 1e-3) / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                            "sample": f"the reference's call pattern restated with torch: {B} copies out ({r_exp:.3f} ms), "
+                                      f"{3 * B * cpr} synchronous chunk copies back ({r_imp:.3f} ms)"}}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -248,11 +317,11 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap", "assist"],
                     help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
                          "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB); "
                          "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters; "
-                         "swap = adapter swap-in from pinned host memory")
+                         "swap = adapter swap-in from pinned host memory; assist = CPU-assist transport")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -281,6 +350,8 @@ def main():
         return bench_c4(args, dev)
     if args.workload == "swap":
         return bench_swap(args, dev)
+    if args.workload == "assist":
+        return bench_assist(args, dev)
     return bench_decode(args, dev)
 
 

@@ -119,6 +119,33 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
                        int elt_bytes, void *stream);
 
 /*
+ * CPU-assist transport: the GPU side of the path on which host workers compute the LoRA delta while an
+ * adapter is still loading (HIP equivalents of the reference's tensor_cp copy family,
+ * csrc/cuda_ops.hpp:109-229; no arithmetic here -- the workers are the reference's own processes or any
+ * other host code that follows the slot and signal protocol).
+ *   mlora_host_alloc / mlora_host_free: pinned host memory mapped into the device address space
+ *       (replaces cudaHostRegister of the shared-memory segments, cuda_ops.hpp:109-112); *dev_ptr is the
+ *       address kernels use, *host_ptr the one the workers use.  Zero-filled.
+ *   mlora_assist_export: hidden [B * tkn, H] (device, 16-bit) -> x_slots [n_slots, slot_tokens, H], request b
+ *       at slot b, tokens from row 0; then signals[q][w] = sig_base + sig_stride * q + w for the
+ *       B * ceil(tkn / cap) workers of each of the n_proj projections (worker w serves request
+ *       w / ceil(tkn / cap), tokens [(w mod ceil(tkn / cap)) * cap, ...)).  One launch for the data, one for
+ *       the signals after it.  Replaces Lora_CPU.invoke_lora_async (lora_cpu.py:138-185), codes 2 / 202 / 402.
+ *   mlora_assist_import: for projection q, out_slots[q] [n_slots, slot_tokens, H] -> res[q] [B, tkn, out_size],
+ *       columns [col0, col0 + out_size) of every row (the rank's share under tensor parallelism).  The
+ *       caller launches it once the workers have reset their signals to 0.  Replaces the per-chunk
+ *       cudaHtoD2D calls of Lora_CPU.collect_qkv (lora_cpu.py:187-276).
+ * x_slots, signals and out_slots are DEVICE addresses of mapped host memory (mlora_host_alloc).
+ */
+int mlora_host_alloc(int64_t bytes, void **host_ptr, void **dev_ptr);
+int mlora_host_free(void *host_ptr);
+int mlora_assist_export(const void *hidden, int B, int tkn, int H, void *x_slots, int n_slots, int slot_tokens,
+                        int16_t *signals, int n_proj, int n_workers, int cap, int sig_base, int sig_stride,
+                        void *stream);
+int mlora_assist_import(int n_proj, void *const *res, const void *const *out_slots, int B, int tkn, int H,
+                        int out_size, int col0, int n_slots, int slot_tokens, void *stream);
+
+/*
  * Decode (BGMV): for every token t with adapter a = tok_adapter[t] and every projection p
  *     y_p[t] = (accumulate ? y_p[t] : 0) + scaling[a] * (x_p[t] . A_{p,a}) . B_{p,a}
  * shrink and expand fused in one launch, rank-r intermediate kept on chip in fp32.
