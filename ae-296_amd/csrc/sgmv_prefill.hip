@@ -339,8 +339,9 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p)
     constexpr int NBC = TN / 16;               // 16-column blocks per step
     constexpr int BPITCH = TN * 2 + 16;        // bytes per rank row of the LDS B tile (16-byte aligned rows)
     constexpr int OPITCH = TN + 4;             // floats per token row of the staging tile
-    constexpr int BQ = BT ? 1 : KP * (TN / 8) / SG_NT;   // B-tile loads per thread and step
-    __shared__ __attribute__((aligned(16))) unsigned char s_b[BT ? 16 : KP * BPITCH];
+    constexpr int TPITCH = KP * 2 + 16;        // reference layout: bytes per output column of the LDS tile (K contiguous)
+    constexpr int BQ = KP * (TN / 8) / SG_NT;  // B-tile loads per thread and step (either layout: KP x TN values)
+    __shared__ __attribute__((aligned(16))) unsigned char s_b[BT ? TN * TPITCH : KP * BPITCH];
     __shared__ __attribute__((aligned(16))) float s_out[SG_NT / 64][16][OPITCH];
     __shared__ int s_brow[BT ? 1 : KP];
     typedef __attribute__((address_space(3))) volatile float lds_vfloat;
@@ -426,6 +427,16 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p)
                 const int col = col0 + c * 8;
                 b_nx[q] = (row >= 0 && col < col_end) ? ldg16(brows + (size_t)row * hout + col) : zero16();
             }
+        } else {
+            // reference layout: column c of the adapter's [hout, r] block holds its r values contiguously, so
+            // the tile of TN columns is one contiguous run when r = KP; 16-byte chunk (column, 8 ranks) per load
+#pragma unroll
+            for (int q = 0; q < BQ; q++) {
+                const int e = tid + q * SG_NT;
+                const int cl = e / (KP / 8), k0 = (e - cl * (KP / 8)) * 8;
+                const int col = col0 + cl;
+                b_nx[q] = (col < col_end && k0 < r) ? ldg16(bt + (size_t)col * r + k0) : zero16();
+            }
         }
     };
     prefetch(col_begin);
@@ -442,6 +453,16 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p)
                 const int e = tid + q * SG_NT;
                 const int j = e / (TN / 8), c = e - j * (TN / 8);
                 *reinterpret_cast<uint4 *>(s_b + j * BPITCH + c * 16) = b_nx[q];
+            }
+            __syncthreads();
+        } else {
+            // park the tile column-major (K contiguous per column): exactly the in-lane order the MFMA wants
+            __syncthreads();
+#pragma unroll
+            for (int q = 0; q < BQ; q++) {
+                const int e = tid + q * SG_NT;
+                const int cl = e / (KP / 8), kc = e - cl * (KP / 8);
+                *reinterpret_cast<uint4 *>(s_b + cl * TPITCH + kc * 16) = b_nx[q];
             }
             __syncthreads();
         }
@@ -464,9 +485,7 @@ __global__ __launch_bounds__(SG_NT) void sgmv_expand_kernel(const SgmvArgs p)
                     bop = make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
                                      __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
                 } else {
-                    const int col = col0 + nb * 16 + m;
-                    const int k0 = ks * 32 + 8 * g;
-                    bop = (col < col_end && k0 < r) ? ldg16(bt + (size_t)col * r + k0) : zero16();
+                    bop = *reinterpret_cast<const uint4 *>(s_b + (nb * 16 + m) * TPITCH + (ks * 4 + g) * 16);
                 }
                 // D[token 4g+i][column m of the block]: A operand = V, B operand = B
                 acc[nb] = mfma16<DT>(vhi[ks], bop, acc[nb]);
