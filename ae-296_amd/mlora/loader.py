@@ -10,7 +10,7 @@ shared memory (``shared_tensor.py:111-154``: layers 8..31 first, code 2 after la
 
 Here an adapter is staged once in pinned host memory, layer-major; a load allocates the slot's
 pages (a page-table update), then for each group of layers issues one host->device copy into a
-staging buffer and one scatter launch per layer that places the rank rows on the slot's pages
+staging buffer and scatter launches (as many layers per launch as the job table holds) that place the rank rows on the slot's pages
 (``mlora_pool_scatter``), all on a copy stream of default priority, with an event per group.  A
 consumer asks ``ticket.ready(layer)`` (event query, no synchronisation) or makes its own stream
 wait for exactly the layers it is about to read (``ticket.wait_layer``).
@@ -93,7 +93,7 @@ class LoadTicket:
 
 
 class AdapterLoader:
-    def __init__(self, pool: AdapterPool, layers_per_copy: int = 4, first_layer: int = 8):
+    def __init__(self, pool: AdapterPool, layers_per_copy: int = 8, first_layer: int = 8):
         if 2 * len(pool.projections) > _ext.SCATTER_MAX_JOBS:
             raise ValueError(f"at most {_ext.SCATTER_MAX_JOBS // 2} projections per pool")
         self.pool = pool
@@ -156,16 +156,21 @@ class AdapterLoader:
                         start = i
                 for l0, l1 in runs:
                     self._staging[l0:l1, :layer_elems].copy_(host.blob[l0:l1], non_blocking=True)
-                for layer in group:
+                # as many layers per scatter launch as the job table holds
+                per_launch = max(1, _ext.SCATTER_MAX_JOBS // (2 * len(self.projs)))
+                for i0 in range(0, len(group), per_launch):
                     src, dst, width = _VoidArr(), _VoidArr(), _IntArr()
-                    base = self._staging[layer].data_ptr()
-                    for i, p in enumerate(self.projs):
-                        hin, hout = pool.projections[p]
-                        a0, b0 = host.offsets[p]
-                        a_ptr, b_ptr = pool.slab_ptrs(layer, p)
-                        src[2 * i], dst[2 * i], width[2 * i] = base + a0 * esz, a_ptr, hin
-                        src[2 * i + 1], dst[2 * i + 1], width[2 * i + 1] = base + b0 * esz, b_ptr, hout
-                    rc = lib.mlora_pool_scatter(2 * len(self.projs), src, dst, width, pages_c, len(page_ids), host.rank,
+                    n_jobs = 0
+                    for layer in group[i0:i0 + per_launch]:
+                        base = self._staging[layer].data_ptr()
+                        for p in self.projs:
+                            hin, hout = pool.projections[p]
+                            a0, b0 = host.offsets[p]
+                            a_ptr, b_ptr = pool.slab_ptrs(layer, p)
+                            src[n_jobs], dst[n_jobs], width[n_jobs] = base + a0 * esz, a_ptr, hin
+                            src[n_jobs + 1], dst[n_jobs + 1], width[n_jobs + 1] = base + b0 * esz, b_ptr, hout
+                            n_jobs += 2
+                    rc = lib.mlora_pool_scatter(n_jobs, src, dst, width, pages_c, len(page_ids), host.rank,
                                                 pool.page_rows, pool.n_pages, esz, self.stream.cuda_stream)
                     _ext.check(rc)
                 ev = torch.cuda.Event()

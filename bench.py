@@ -173,7 +173,7 @@ def bench_swap(args, dev):
     L, H, r = 32, 4096, 64
     projections = {p: (H, H) for p in "qkv"}
     pool = mlora.AdapterPool(L, projections, n_slots=4, n_pages=64, page_rows=8, max_rank=r, dtype=torch.float16, device=dev)
-    loader = mlora.AdapterLoader(pool, layers_per_copy=args.layers if args.layers > 0 else 4, first_layer=8)
+    loader = mlora.AdapterLoader(pool, layers_per_copy=args.layers if args.layers > 0 else 8, first_layer=8)
     gen = torch.Generator().manual_seed(3003)
     w = {p: (torch.randn(L, H, r, generator=gen) * 0.001, torch.randn(L, r, H, generator=gen) * 0.001) for p in "qkv"}
     host = loader.stage(w, r, 0.5)
