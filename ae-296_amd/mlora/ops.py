@@ -64,11 +64,27 @@ class DecodePlan:
         return self.tok_adapter.numel()
 
 
+N_CUS = 256       # compute units of the device the kernels are written for
+
+
 def default_group(T: int) -> int:
-    """Tokens of one adapter per decode work item when the caller does not say: 2 for small batches
-    (few tokens share an adapter, and the lighter kernels start faster), 4 otherwise (measured:
-    8.3 vs 10.1 us per call at 32 tokens, 21.3 vs 23.5 us at 256)."""
-    return 2 if T <= 64 else 4
+    """Tokens of one adapter per decode work item when the caller does not say: 1 up to 64 tokens and
+    2 up to 128 (the batch then fits one workgroup per compute unit and runs as the single fused launch,
+    see `decode_fused`), 4 beyond (measured per call, three projections: 8.5 us at 64 tokens against
+    9.9 for the two-launch form, 10.8 against 13.2 at 128, 20.5 against 20.9 with 2 at 256)."""
+    return 1 if T <= 64 else 2 if T <= 128 else 4
+
+
+def decode_fused(T: int, group: int, n_proj: int, n_slots: int) -> bool:
+    """Form of a planned decode call when the caller does not say: the single fused launch while its
+    work items, one 512-thread workgroup each, fit the device in one round (the call is then bound by
+    the dependent loads of one workgroup, and a second launch only adds to that); the shrink and expand
+    launches beyond, where spreading one item over many workgroups is what fills the memory system.
+    The item count is the host's estimate: groups of two leave one odd item for about every other adapter."""
+    if group > 2:
+        return False
+    items = T if group == 1 else (T + 1) // 2 + min(T, n_slots) // 2
+    return items * n_proj <= N_CUS
 
 
 def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: Optional[int] = None, per_token: bool = False,
@@ -119,8 +135,8 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     ys[p][t] (+)= scaling[a] * (xs[p][t] . A_{p,a}) . B_{p,a},  a = tok_adapter[t].
 
     With a plan the call runs as a shrink launch and an expand launch over column slices
-    (``fused=False``, the default) or as one fused launch (``fused=True``); without a plan it is
-    always the fused launch with one token per work item.  The two-launch form keeps its fp32
+    (``fused=False``) or as one fused launch (``fused=True``), by default whichever `decode_fused`
+    names for the batch; without a plan it is always the fused launch with one token per work item.  The two-launch form keeps its fp32
     intermediate in a buffer owned by the plan, allocated on the first call that needs it (so
     run one call before capturing a HIP graph); calls that share a plan must therefore follow each
     other on one stream, not overlap on several."""
@@ -146,7 +162,7 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     if plan is not None and plan.T != T:
         raise ValueError("plan was built for a different batch size")
     if fused is None:
-        fused = plan is None
+        fused = plan is None or decode_fused(T, plan.group, n, pool.n_slots)
     if not fused and plan is None:
         raise ValueError("the two-launch form needs a plan")
     ws, ws_bytes = None, 0

@@ -311,6 +311,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
     ap.add_argument("--group", type=int, default=-1,
                     help="tokens of one adapter per work item (0 = no plan, one token each; default: by batch size)")
+    ap.add_argument("--split", action="store_true", help="decode: force the shrink + expand pair also where the host layer would pick the fused launch")
     ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
                          "instead of one call over the seven")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
@@ -419,7 +420,8 @@ def bench_decode(args, dev):
     xs = [{i: torch.randn(T, width[i], device=dev, generator=gen).half() for i in inputs} for _ in range(L)]
     ys = [[torch.randn(T, shapes[p][1], device=dev, generator=gen).half() for p in projs] for _ in range(L)]
     plan = mlora.plan_decode(tok, pool, group=args.group) if args.group else None
-    fused = bool(args.fused or plan is None)
+    fused = bool(args.fused or plan is None or
+                 (not args.split and mlora.ops.decode_fused(T, args.group, len(projs), pool.n_slots)))
 
     # config 5 carries prefill segments through SGMV in the same step (activations shared by the layers:
     # they are larger than the last-level cache anyway)

@@ -32,7 +32,7 @@ def _run(pp, x_bits, tok, y0_bits, group, accumulate=True, fused=None):
 
 
 # launch forms: (group, fused); group 0 = no plan, one token per work item
-FORMS = [(0, True), (1, True), (4, True), (1, False), (2, False), (4, False)]
+FORMS = [(0, True), (1, True), (2, True), (4, True), (1, False), (2, False), (4, False)]
 
 
 CASES = [
@@ -99,6 +99,29 @@ def test_bgmv_integer_inputs_bit_exact(group, fused):
     say(f"bgmv integer-valued inputs group={group} fused={fused}")
     got = _run(pp, x, tok, y0, group, fused=fused)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("T,want_group,want_fused", [(48, 1, True), (100, 2, True), (300, 4, False)])
+def test_bgmv_default_form_by_batch_size(T, want_group, want_fused):
+    """Without `group` and `fused` the host layer picks them from the batch size; the result is the
+    explicitly requested form's, bit for bit, and meets the oracle's tolerance."""
+    from mlora import ops
+    rng = np.random.default_rng(300 + T)
+    pp = PagedPool(rng, [16] * 12, 1024, 1024, page_rows=8, dtype=FP16)
+    tok = rng.integers(0, 12, T).astype(np.int32)
+    x = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
+    y0 = bits_of(rng.standard_normal((T, 1024)).astype(np.float32), FP16)
+    pool = upload_pool(pp)
+    t = torch.from_numpy(tok).cuda()
+    plan = plan_decode(t, pool)
+    assert plan.group == want_group and ops.decode_fused(T, plan.group, 1, pool.n_slots) == want_fused
+    say(f"bgmv default form T={T}")
+    y = bits_to_torch(y0, FP16, "cuda")
+    bgmv([y], [bits_to_torch(x, FP16, "cuda")], pool, 0, ["p"], t, plan=plan)
+    torch.cuda.synchronize()
+    got = torch_to_bits(y)
+    assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16, f"default form T={T}")
+    assert np.array_equal(got, _run(pp, x, tok, y0, want_group, fused=want_fused))
 
 
 def test_bgmv_tokens_without_adapter_and_rank_tails():

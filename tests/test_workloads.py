@@ -44,3 +44,13 @@ def test_zipf_adapters_range_and_skew():
     assert a.dtype == np.int32 and a.min() >= 0 and a.max() < 64
     counts = np.sort(np.bincount(a, minlength=64))[::-1]
     assert counts[0] > 4 * counts[16]          # p_1 / p_17 = 17 under Zipf(1.0)
+
+
+def test_decode_form_follows_the_batch_size():
+    from mlora import ops
+    assert [ops.default_group(t) for t in (1, 32, 64, 65, 128, 129, 256, 4096)] == [1, 1, 1, 2, 2, 4, 4, 4]
+    # one work item per workgroup, one workgroup per compute unit: fused while that holds
+    assert ops.decode_fused(64, 1, 3, 16) and ops.decode_fused(64, 1, 4, 16) and not ops.decode_fused(64, 1, 5, 16)
+    assert ops.decode_fused(128, 2, 3, 32) and not ops.decode_fused(192, 2, 3, 48)
+    assert not ops.decode_fused(128, 2, 3, 128)          # every token its own adapter: 128 items per projection
+    assert not ops.decode_fused(8, 4, 1, 8) and not ops.decode_fused(8, 8, 1, 8)
