@@ -523,6 +523,65 @@ int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x, c
                        workspace_bytes, mlora::SGMV_APPLY, stream);
 }
 
+int mlora_gemm_lora_planned(int n_proj, void *const *y, const void *const *x, const void *const *w,
+                            const void *const *a_rows, const void *const *b_rows, const int32_t *hin,
+                            const int32_t *hout, const int32_t *seg_start, const int32_t *seg_len,
+                            const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl, const int32_t *rank,
+                            const float *scaling, int T, int n_adapters, int max_pages, int page_rows,
+                            int64_t n_pages, int max_rank, int dtype, void *workspace, int64_t workspace_bytes,
+                            void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (T < 0 || n_seg < 0) return fail(MLORA_EINVAL, "T and n_seg must be >= 0 (got %d, %d)", T, n_seg);
+    if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
+    if (T == 0) return MLORA_OK;
+    if (!y || !x || !w || !hin || !hout) return fail(MLORA_EINVAL, "per-projection arrays must not be NULL");
+    const bool lora = n_seg > 0;
+    if (lora && (!a_rows || !b_rows || !seg_start || !seg_len || !seg_adapter)) return fail(MLORA_EINVAL, "NULL pointer for a call with segments");
+    mlora::SgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    mlora::GemmLoraArgs g;
+    memset(&g, 0, sizeof(g));
+    int rc;
+    if (lora) {
+        rc = check_pool(a.pool, page_tbl, rank, scaling, n_adapters, max_pages, page_rows, n_pages, max_rank);
+        if (rc) return rc;
+    }
+    a.n_proj = n_proj;
+    for (int p = 0; p < n_proj; p++) {
+        if (!y[p] || !x[p] || !w[p] || (lora && (!a_rows[p] || !b_rows[p]))) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
+        rc = check_dims(hin[p], hout[p]);
+        if (rc) return rc;
+        if (!aligned16(y[p]) || !aligned16(x[p]) || !aligned16(w[p]) || (lora && (!aligned16(a_rows[p]) || !aligned16(b_rows[p]))))
+            return fail(MLORA_EALIGN, "projection %d: device pointers must be 16-byte aligned", p);
+        // the kernel addresses a weight through one buffer descriptor with 32-bit offsets
+        if ((int64_t)hin[p] * hout[p] * 2 >= (1LL << 32)) return fail(MLORA_ERANGE, "projection %d: base weight of 4 GiB or more", p);
+        if ((int64_t)256 * hin[p] * 2 >= (1LL << 32)) return fail(MLORA_ERANGE, "projection %d: hin too large", p);
+        a.pr[p].y = y[p]; a.pr[p].x = x[p]; a.pr[p].hin = hin[p]; a.pr[p].hout = hout[p];
+        g.pr[p].y = y[p]; g.pr[p].x = x[p]; g.pr[p].w = w[p]; g.pr[p].hin = hin[p]; g.pr[p].hout = hout[p];
+        if (lora) { a.pr[p].a_rows = a_rows[p]; a.pr[p].b_rows = b_rows[p]; g.pr[p].b_rows = b_rows[p]; }
+    }
+    g.n_proj = n_proj; g.T = T; g.lora = lora ? 1 : 0;
+    if (lora) {
+        const SgmvWs ws = sgmv_layout(T, n_seg, n_proj);
+        if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
+        if (workspace_bytes < (int64_t)ws.total)
+            return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)ws.total);
+        a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter; a.n_seg = n_seg;
+        a.T = T; a.accumulate = 0; a.b_transposed = 0; a.seg_uniform_len = 0;
+        carve(a, workspace, ws);
+        rc = mlora::launch_sgmv(a, dtype, max_rank, mlora::SGMV_SHRINK, static_cast<hipStream_t>(stream));
+        if (rc) return fail(MLORA_ELAUNCH, "shrink launch failed: %s", hipGetErrorString((hipError_t)rc));
+        for (int p = 0; p < n_proj; p++) {
+            g.pr[p].v = a.pr[p].v; g.pr[p].vhi = a.pr[p].vhi; g.pr[p].vlo = a.pr[p].vlo; g.pr[p].ksplit = a.pr[p].ksplit;
+        }
+        g.tile_rec = a.tile_rec; g.n_tiles = a.n_tiles; g.max_tiles = a.max_tiles; g.n_rows_b = a.pool.n_rows_b;
+    }
+    rc = mlora::launch_gemm_lora(g, dtype, lora ? max_rank : 16, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "gemm launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
 int mlora_prefill_reflayout(void *y, const void *x, const void *A_T, const void *B_T, int B, int Lpad, int L,
                             int r, int hin, int hout, int layer_idx, int dtype, void *workspace,
                             int64_t workspace_bytes, void *stream)

@@ -1,0 +1,457 @@
+// Base projection with the LoRA expand folded in, for gfx950 (prefill: packed tokens, one adapter per segment):
+//     y[t, :] = round16( x[t, :] . W  +  s_a * (x[t, :] . A_a) . B_a )
+// W is [hin, hout] row-major (the layout lightllm keeps its projection weights in:
+// lightllm/models/llama/layer_weights/transformer_layer_weight.py:44-46), x is [T, hin].
+// Replaces, for one layer, torch.mm(x, W) followed by `q += q_lora`
+// (lightllm/models/llama/layer_infer/transformer_layer_infer.py:145-147,160-171): y is written once and
+// never read, x is read once per column tile.
+//
+// The rank-r intermediate s_a * (x . A_a) comes from the SGMV shrink launch (sgmv_prefill.hip) and the
+// scaled reduce below, as a hi + lo pair of 16-bit values per element; the kernel here treats it as
+// extra K columns of the GEMM: after the K loop over W, every 32-row block of the output tile runs
+// rank / 16 more MFMA steps with (intermediate, B rows of its adapter) as operands.
+//
+// One workgroup (256 threads, 2 x 2 wavefronts of 128 x 128 outputs each) computes a 256 x 256 tile of y
+// on v_mfma_f32_32x32x16_{f16,bf16}.  K advances 64 columns per step through two LDS stages: while the
+// MFMAs of step k run from one stage, the registers holding step k+1 are parked in the other and the
+// global loads of step k+2 are in flight.  x is K-contiguous, so its operand is a plain 16-byte LDS read;
+// W is N-contiguous and is read back with the transposing LDS read.
+#include "mlora_args.hpp"
+#include "mlora_dev.hpp"
+#include <type_traits>
+
+namespace mlora {
+
+constexpr int GM = 256;                 // rows (tokens) per tile
+constexpr int GN = 256;                 // output columns per tile
+constexpr int GK = 64;                  // K columns per stage
+constexpr int G_NT = 256;
+constexpr int PB = GN * 2 + 64;         // LDS pitch of a parked B row (expand step): the 4 rows x 32 bytes of a transposing read fall on distinct banks
+constexpr int A_BYTES = GM * GK * 2;    // x tile of a stage, rows unpadded and chunk-swizzled
+constexpr int B_BYTES = GK * GN * 2;    // W tile of a stage, likewise
+constexpr int STAGE = A_BYTES + B_BYTES;
+constexpr int OPITCH = 128 * 2 + 16;    // bytes per row of a wavefront's 32 x 128 output staging tile
+constexpr int GROUP_M = 4;              // row tiles that share W column tiles back to back on one XCD
+typedef short gl_short4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) gl_short4 gl_lds_short4;
+
+static_assert(2 * STAGE <= 160 * 1024 - 4096, "two stages and the small tables must fit the LDS of a compute unit");
+static_assert(4 * 32 * OPITCH <= STAGE && MAX_RANK * PB <= STAGE, "output staging and the parked B rows reuse a stage");
+
+template <int DT>
+__device__ __forceinline__ float16_t mfma32(const uint4 &a, const uint4 &b, float16_t c)
+{
+    if constexpr (DT == DT_F16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
+}
+
+// B operand of a 32x32x16 MFMA out of a row-major [k][n] LDS tile: lane (n = lane % 32, k group = lane / 32)
+// needs rows k0 + 8 * (lane / 32) + 0..7 of column n0 + lane % 32.  Each transposing read serves a 16-lane
+// group: lane i of the group addresses row i / 4, columns 4 * (i % 4) .. + 3, and receives the four rows of
+// column i.
+__device__ __forceinline__ uint4 lds_b_operand(const unsigned char *tile, int pitch, int k0, int n0, int lane)
+{
+    const int g = lane >> 4, m = lane & 15;
+    const unsigned char *src = tile + (k0 + 8 * (g >> 1) + (m >> 2)) * pitch + (n0 + (g & 1) * 16 + (m & 3) * 4) * 2;
+    const gl_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)src);
+    const gl_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)(src + 4 * pitch));
+    return make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
+                      __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
+}
+
+// ------------------------------------------------------------------ scaled reduce
+// vhi + vlo [t][0..RMAX) = s_a * sum over the K splits of the shrink partials, for the tokens of one plan
+// tile (the scaling is folded in here because the GEMM accumulators also hold the base product).
+template <int DT, int RMAX>
+__global__ __launch_bounds__(256) void gemm_lora_reduce_kernel(const GemmLoraArgs p)
+{
+    constexpr int CPT = RMAX / 8;
+    const int tile = blockIdx.x;
+    if (tile >= p.n_tiles[0]) return;
+    const GemmProj &pj = p.pr[blockIdx.y];
+    const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
+    const int ntok = rec[0], adapter = rec[1], tok0 = rec[4];
+    if (adapter < 0 || ntok <= 0 || tok0 < 0 || tok0 + ntok > p.T) return;
+    const float scale = __builtin_bit_cast(float, rec[3]);
+    for (int idx = threadIdx.x; idx < ntok * CPT; idx += 256) {
+        const int t = tok0 + idx / CPT, c0 = (idx % CPT) * 8;
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = 0.f;
+        for (int sp = 0; sp < pj.ksplit; sp++) {
+            const float4_t *vp = reinterpret_cast<const float4_t *>(pj.v + ((size_t)sp * p.T + t) * MAX_RANK + c0);
+            const float4_t a = vp[0], b = vp[1];
+            v[0] += a[0]; v[1] += a[1]; v[2] += a[2]; v[3] += a[3];
+            v[4] += b[0]; v[5] += b[1]; v[6] += b[2]; v[7] += b[3];
+        }
+        uint32_t h[8], l[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float sv = scale * v[e];
+            h[e] = cvt16<DT>(sv);
+            l[e] = cvt16<DT>(sv - lo_f32<DT>(h[e]));
+        }
+        stg16(pj.vhi + (size_t)t * MAX_RANK + c0,
+              make_uint4(h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)));
+        stg16(pj.vlo + (size_t)t * MAX_RANK + c0,
+              make_uint4(l[0] | (l[1] << 16), l[2] | (l[3] << 16), l[4] | (l[5] << 16), l[6] | (l[7] << 16)));
+    }
+}
+
+// ------------------------------------------------------------------ GEMM + expand
+template <int DT>
+__global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p)
+{
+    // two stages as two arrays: the compiler then knows that parking step k + 1 cannot alias the operand reads of step k
+    __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char smem1[STAGE];
+    __shared__ unsigned long long s_mask[G_NT / 64];
+
+    // ---- which projection, which tile.  Workgroups go to the 8 XCDs round-robin by id; every XCD works
+    // through one contiguous range of the tile order below, in which GROUP_M row tiles sweep the column
+    // tiles together, so that the tiles in flight on one XCD (one L2) share their x and W panels.
+    int proj = 0;
+    while (proj + 1 < p.n_proj && blockIdx.x >= p.pr[proj].end) proj++;
+    const GemmProj &pj = p.pr[proj];
+    const int w = (int)(blockIdx.x - (proj ? p.pr[proj - 1].end : 0u));
+    const int ntn = pj.ntn, ntm = p.ntm;
+    const int n_tiles_out = ntm * ntn;
+    const int per_xcd = (n_tiles_out + 7) >> 3;
+    const int L = (w & 7) * per_xcd + (w >> 3);
+    if ((w >> 3) >= per_xcd || L >= n_tiles_out) return;
+    const int grp = L / (GROUP_M * ntn), within = L - grp * (GROUP_M * ntn);
+    const int rows_in_grp = ntm - grp * GROUP_M < GROUP_M ? ntm - grp * GROUP_M : GROUP_M;
+    const int mt = grp * GROUP_M + within % rows_in_grp, nt = within / rows_in_grp;
+    const int m0 = mt * GM, n0 = nt * GN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int T = p.T, hin = pj.hin, hout = pj.hout;
+    const uint16_t *__restrict__ x = static_cast<const uint16_t *>(pj.x);
+    const uint16_t *__restrict__ wgt = static_cast<const uint16_t *>(pj.w);
+
+    // ---- global -> LDS, without passing through registers (buffer_load ... lds): each such load moves
+    // 64 lanes x 16 bytes into 1 KiB of consecutive LDS, lane i to slot i.  The tiles therefore have no row
+    // padding; bank conflicts are avoided by storing 16-byte chunk c of a row at position c ^ key(row), which
+    // costs nothing on the way in (lane i simply fetches the chunk that belongs in slot i).
+    //   x tile [256 rows][8 chunks]:  key = (row / 2) % 8   (16 operand rows of one chunk column -> 16 bank groups)
+    //   W tile [64 k rows][32 chunks]: key = (k % 4) * 4     (the 4 rows of a transposing read -> 4 bank groups)
+    // One load of wavefront w covers 8 rows of x (rows 8 (4 q + w) ..) or 2 rows of W (rows 2 (4 q + w) ..).
+    // Rows beyond T and columns beyond hout are clamped to valid addresses; what they produce is never stored.
+    const int rows_here = T - m0 < GM ? T - m0 : GM;
+    unsigned aoff[8], boff[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int row = 8 * (4 * q + wave) + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        const int r = row < rows_here ? row : rows_here - 1;
+        aoff[q] = ((unsigned)r * (unsigned)hin + (unsigned)c * 8u) * 2u;
+    }
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int k = 2 * (4 * q + wave) + (lane >> 5);
+        const int c = (lane & 31) ^ ((k & 3) << 2);
+        int col = n0 + c * 8;
+        col = col < hout ? col : hout - 8;
+        boff[q] = ((unsigned)k * (unsigned)hout + (unsigned)col) * 2u;
+    }
+    // A uniform descriptor per operand, a fixed 32-bit offset per load in a VGPR and the K advance as the scalar
+    // offset: the loop spends no vector instructions on addresses.  The x descriptor starts at this tile's first
+    // row; the launcher guarantees hin * hout * 2 < 4 GiB.
+    const size_t x_bytes = (size_t)rows_here * hin * 2;
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(x + (size_t)m0 * hin), (short)0, (int)(x_bytes < 0xffffffffu ? x_bytes : 0xffffffffu), 0x00020000);
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint16_t *>(wgt), (short)0, (int)((size_t)hin * hout * 2), 0x00020000);
+    typedef __attribute__((address_space(3))) void lds_void;
+    auto dma_a = [&](unsigned char *stage, int kt) {
+        const unsigned soff = (unsigned)kt * (GK * 2);
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(xrs, (lds_void *)(stage + (4 * q + wave) * 1024), 16, (int)aoff[q], (int)soff, 0, 0);
+    };
+    auto dma_b = [&](unsigned char *stage, int kt) {
+        const unsigned soff = (unsigned)kt * GK * (unsigned)hout * 2u;
+#pragma unroll
+        for (int q = 0; q < 8; q++)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(wrs, (lds_void *)(stage + A_BYTES + (4 * q + wave) * 1024), 16, (int)boff[q], (int)soff, 0, 0);
+    };
+
+    float16_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    // Operand addresses inside a stage.  x: lane (row wm * 128 + 32 i + lane % 32, chunk 2 kk + lane / 32); the key
+    // of the row does not depend on i.  W: lane group g = lane / 16, m = lane % 16 reads rows 16 kk + 8 (g / 2) +
+    // m / 4 (+ 4), bytes of columns wn * 128 + 32 j + 16 (g % 2) + 4 (m % 4) ..; the key (m / 4) * 4 flips bits of j.
+    unsigned a_at[4], b_at[4];
+    {
+        const int row = wm * 128 + l32, key = (l32 >> 1) & 7;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) a_at[kk] = (unsigned)(row * (GK * 2) + (((2 * kk + lh) ^ key) << 4));
+        const int g = lane >> 4, m = lane & 15;
+        const int krow = 8 * (g >> 1) + (m >> 2);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int c = wn * 16 + ((j ^ (m >> 2)) << 2) + (g & 1) * 2 + ((m & 3) >> 1);
+            b_at[j] = (unsigned)(A_BYTES + krow * (GN * 2) + c * 16 + (m & 1) * 8);
+        }
+    }
+    // Operands of one K = 16 step (4 x fragments, 4 W fragments), read one step ahead of the MFMAs that use them.
+    uint4 fa[2][4], fb[2][4];
+    auto frags = [&](const unsigned char *stage, auto kk_c, uint4 (&af)[4], uint4 (&bf)[4]) {
+        constexpr int kk = decltype(kk_c)::value;
+#pragma unroll
+        for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(stage + a_at[kk] + i * 32 * (GK * 2));
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const unsigned char *src = stage + b_at[j] + kk * 16 * (GN * 2);
+            const gl_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)src);
+            const gl_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)(src + 4 * (GN * 2)));
+            bf[j] = make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
+                               __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
+        }
+    };
+    auto mfma16x = [&](const uint4 (&af)[4], const uint4 (&bf)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = mfma32<DT>(af[i], bf[j], acc[i][j]);
+    };
+    using K0 = std::integral_constant<int, 0>;
+    using K1 = std::integral_constant<int, 1>;
+    using K2 = std::integral_constant<int, 2>;
+    using K3 = std::integral_constant<int, 3>;
+#define GL_FENCE() __builtin_amdgcn_sched_barrier(0)
+    // Scheduling hints: one MFMA, then at most one operand read and at most one global load, so that the memory
+    // instructions issue in the shadow of the MFMAs instead of in a burst between them (an MFMA occupies its pipe
+    // for 32 cycles, issuing it takes 4).
+#define GL_MIX(n_ds_read, n_load)                                                  \
+    _Pragma("unroll") for (int n_ = 0; n_ < 16; n_++) {                              \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                          \
+        if (n_ < (n_ds_read)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    \
+        if (n_ < (n_load)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);       \
+    }
+    // One K step of 64 columns out of stage `cur`, four slices of 16.  Operand reads run one slice ahead of
+    // the MFMAs.  The barrier sits before the last slice: by then every wavefront has read all it needs from
+    // `cur` and the loads of step kt + 1 (requested a whole step earlier) have landed in the other stage, so the
+    // last slice's operand prefetch reads the other stage, and `cur` is free to receive step kt + 2 at once.
+    auto k_step = [&](auto cur_c, auto has1_c, auto has2_c, int kt) {
+        constexpr int cur_i = decltype(cur_c)::value;
+        constexpr bool has1 = decltype(has1_c)::value, has2 = decltype(has2_c)::value;
+        unsigned char *cur = cur_i ? smem1 : smem, *nxt = cur_i ? smem : smem1;
+        frags(cur, K1{}, fa[1], fb[1]);
+        mfma16x(fa[0], fb[0]);
+        GL_MIX(12, 0)
+        GL_FENCE();
+        frags(cur, K2{}, fa[0], fb[0]);
+        mfma16x(fa[1], fb[1]);
+        GL_MIX(12, 0)
+        GL_FENCE();
+        frags(cur, K3{}, fa[1], fb[1]);
+        mfma16x(fa[0], fb[0]);
+        GL_MIX(12, 0)
+        GL_FENCE();
+        __syncthreads();
+        if constexpr (has2) { dma_a(cur, kt + 2); dma_b(cur, kt + 2); }
+        if constexpr (has1) frags(nxt, K0{}, fa[0], fb[0]);
+        mfma16x(fa[1], fb[1]);
+        GL_MIX(12, 16)
+        GL_FENCE();
+    };
+    using St0 = std::integral_constant<int, 0>;
+    using St1 = std::integral_constant<int, 1>;
+    using Yes = std::true_type;
+    using No = std::false_type;
+
+    // Full K steps run through the pipeline; a partial last step follows on its own.
+    const int nkf = hin / GK;
+    if (nkf > 0) {
+        dma_a(smem, 0);
+        dma_b(smem, 0);
+        if (nkf > 1) { dma_a(smem1, 1); dma_b(smem1, 1); }
+        __syncthreads();
+        frags(smem, K0{}, fa[0], fb[0]);
+        int kt = 0;
+#pragma unroll 1
+        for (; kt + 4 <= nkf; kt += 2) {                                 // steady state; leaves 2 or 3 steps
+            k_step(St0{}, Yes{}, Yes{}, kt);
+            k_step(St1{}, Yes{}, Yes{}, kt + 1);
+        }
+        if (nkf - kt == 3) { k_step(St0{}, Yes{}, Yes{}, kt); k_step(St1{}, Yes{}, No{}, kt + 1); k_step(St0{}, No{}, No{}, kt + 2); }
+        else if (nkf - kt == 2) { k_step(St0{}, Yes{}, No{}, kt); k_step(St1{}, No{}, No{}, kt + 1); }
+        else k_step(St0{}, No{}, No{}, kt);
+    }
+    if (nkf * GK < hin) {
+        // Partial last K step: through registers, with chunks of x and rows of W beyond hin replaced by zeros,
+        // parked in the same swizzled layout.  Every wavefront has passed the last barrier of the pipeline.
+        const int ncc = hin >> 3;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int row = 8 * (4 * q + wave) + (lane >> 3);
+            const int c = (lane & 7) ^ ((row >> 1) & 7);
+            const bool ok = nkf * 8 + c < ncc;
+            const unsigned back = ok ? 0u : (unsigned)(nkf * 8 + c - (ncc - 1)) * 16u;
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(aoff[q] - back), nkf * (GK * 2), 0);
+            *reinterpret_cast<uint4 *>(smem + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
+        }
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int k = nkf * GK + 2 * (4 * q + wave) + (lane >> 5);
+            const bool ok = k < hin;
+            const unsigned back = ok ? 0u : (unsigned)(k - (hin - 1)) * (unsigned)hout * 2u;
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wrs, (int)(boff[q] - back), (int)((unsigned)nkf * GK * (unsigned)hout * 2u), 0);
+            *reinterpret_cast<uint4 *>(smem + A_BYTES + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
+        }
+        __syncthreads();
+        const int rem = hin - nkf * GK;
+        frags(smem, K0{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]);
+        if (rem > 16) { frags(smem, K1{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
+        if (rem > 32) { frags(smem, K2{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
+        if (rem > 48) { frags(smem, K3{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
+        __syncthreads();
+    }
+#undef GL_FENCE
+#undef GL_MIX
+
+    // ---- LoRA expand as extra K columns.  Plan tiles (at most 64 consecutive tokens of one adapter) that
+    // overlap this row block are found by scanning the tile list, 256 tiles at a time; for each, the B rows
+    // of its adapter for this column tile are parked in LDS and every 32-row block that overlaps the tile
+    // runs rank / 16 MFMA steps with the intermediate of the tile's rows (zero for the other rows).
+    if (p.lora) {
+        const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
+        const int n_plan = p.n_tiles[0];
+        unsigned char *sb = smem;                  // [rank rows][PB]
+        for (int b0 = 0; b0 < n_plan; b0 += G_NT) {
+            const int ti = b0 + tid;
+            bool hit = false;
+            if (ti < n_plan) {
+                const int32_t *rec = p.tile_rec + (size_t)ti * TILE_WORDS;
+                const int ntok = rec[0], tok0 = rec[4];
+                hit = rec[1] >= 0 && rec[2] > 0 && ntok > 0 && tok0 >= 0 && tok0 + ntok <= T && tok0 < m0 + GM && tok0 + ntok > m0;
+            }
+            const unsigned long long bal = __ballot(hit);
+            __syncthreads();                       // s_mask of the previous batch has been consumed
+            if (lane == 0) s_mask[wave] = bal;
+            __syncthreads();
+#pragma unroll 1
+            for (int w4 = 0; w4 < G_NT / 64; w4++) {
+                unsigned long long mask = s_mask[w4];
+#pragma unroll 1
+                while (mask) {
+                    const int cur = b0 + w4 * 64 + __builtin_ctzll(mask);
+                    mask &= mask - 1;
+                    const int32_t *__restrict__ rec = p.tile_rec + (size_t)cur * TILE_WORDS;
+                    const int ntok = rec[0], r = rec[2] < p.rmax ? rec[2] : p.rmax, tok0 = rec[4];
+                    const int kp = (r + 15) & ~15;
+                    const int i0 = tok0 - m0, i1 = tok0 + ntok - m0;      // rows of the block, may stick out on either side
+                    __syncthreads();               // the previous tile's B rows have been consumed
+                    for (int e = tid; e < kp * 32; e += G_NT) {
+                        const int j = e >> 5, c = e & 31;
+                        const int row = rec[TILE_ROWS_AT + j];
+                        const int col = n0 + c * 8;
+                        uint4 v = zero16();
+                        if (row >= 0 && row < p.n_rows_b && col < hout) v = ldg16(brows + (size_t)row * hout + col);
+                        *reinterpret_cast<uint4 *>(sb + j * PB + c * 16) = v;
+                    }
+                    __syncthreads();
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int R0 = wm * 128 + i * 32;
+                        if (R0 + 32 <= i0 || R0 >= i1) continue;          // uniform per wavefront
+                        const int my = R0 + l32;
+                        const bool mine = my >= i0 && my < i1;
+                        const size_t vrow = (size_t)(m0 + (mine ? my : i0 > 0 ? i0 : 0)) * MAX_RANK;
+                        for (int ks = 0; ks < kp; ks += 16) {
+                            uint4 vh = ldg16(pj.vhi + vrow + ks + 8 * lh);
+                            uint4 vl = ldg16(pj.vlo + vrow + ks + 8 * lh);
+                            if (!mine) { vh = zero16(); vl = zero16(); }
+#pragma unroll
+                            for (int j = 0; j < 4; j++) {
+                                const uint4 bf = lds_b_operand(sb, PB, ks, wn * 128 + j * 32, lane);
+                                acc[i][j] = mfma32<DT>(vh, bf, acc[i][j]);
+                                acc[i][j] = mfma32<DT>(vl, bf, acc[i][j]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- y: every wavefront passes its 128 x 128 block through a private LDS tile, 32 rows at a time, so
+    // that the stores are 16 bytes wide and a 16-lane row covers 256 contiguous bytes of one token.
+    // D layout of the 32x32 MFMA: lane holds column lane % 32, rows 8 * (e / 4) + 4 * (lane / 32) + e % 4.
+    // The tile is private to the wavefront and LDS operations of one wavefront complete in order, so no
+    // barrier is needed; the accesses are volatile so that they stay in program order.
+    {
+        unsigned char *so = smem + wave * (32 * OPITCH);
+        typedef __attribute__((address_space(3))) volatile uint16_t lds_vu16;
+        typedef __attribute__((address_space(3))) volatile u32x4_t lds_vu32x4;
+        uint16_t *__restrict__ y = static_cast<uint16_t *>(pj.y);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int row = 8 * (e >> 2) + 4 * lh + (e & 3);
+                    *(lds_vu16 *)(so + row * OPITCH + (j * 32 + l32) * 2) = (uint16_t)cvt16<DT>(acc[i][j][e]);
+                }
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const int pp = lane + 64 * q, row = pp >> 4, c = pp & 15;
+                const u32x4_t v = *(lds_vu32x4 *)(so + row * OPITCH + c * 16);
+                const int gr = m0 + wm * 128 + i * 32 + row, gc = n0 + wn * 128 + c * 8;
+                if (gr < T && gc < hout) stg16_stream(y + (size_t)gr * hout + gc, make_uint4(v.x, v.y, v.z, v.w));
+            }
+        }
+    }
+}
+
+template <int DT, int RMAX>
+static int launch_gl(const GemmLoraArgs &a, hipStream_t s)
+{
+    GemmLoraArgs g = a;
+    g.rmax = RMAX;
+    g.ntm = (g.T + GM - 1) / GM;
+    unsigned end = 0;
+    for (int q = 0; q < g.n_proj; q++) {
+        g.pr[q].ntn = (g.pr[q].hout + GN - 1) / GN;
+        const long long tiles = (long long)g.ntm * g.pr[q].ntn;
+        const long long padded = (tiles + 7) / 8 * 8;
+        if (end + padded > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+        end += (unsigned)padded;
+        g.pr[q].end = end;
+    }
+    if (end == 0) return 0;
+    if (g.lora) {
+        hipLaunchKernelGGL((gemm_lora_reduce_kernel<DT, RMAX>), dim3((unsigned)g.max_tiles, (unsigned)g.n_proj), dim3(256), 0, s, g);
+        const int rc = (int)hipGetLastError();
+        if (rc) return rc;
+    }
+    hipLaunchKernelGGL((gemm_lora_kernel<DT>), dim3(end), dim3(G_NT), 0, s, g);
+    return (int)hipGetLastError();
+}
+
+int launch_gemm_lora(const GemmLoraArgs &a, int dtype, int max_rank, hipStream_t s)
+{
+    if (dtype == DT_F16) {
+        if (max_rank <= 16) return launch_gl<DT_F16, 16>(a, s);
+        if (max_rank <= 32) return launch_gl<DT_F16, 32>(a, s);
+        return launch_gl<DT_F16, 64>(a, s);
+    }
+    if (max_rank <= 16) return launch_gl<DT_BF16, 16>(a, s);
+    if (max_rank <= 32) return launch_gl<DT_BF16, 32>(a, s);
+    return launch_gl<DT_BF16, 64>(a, s);
+}
+
+}  // namespace mlora

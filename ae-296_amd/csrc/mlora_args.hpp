@@ -136,6 +136,34 @@ struct SgmvArgs {
     int max_tiles;
 };
 
+// One projection of a base GEMM + LoRA call.
+struct GemmProj {
+    void *y;               // [T, hout], written once
+    const void *x;         // [T, hin]
+    const void *w;         // [hin, hout] row-major base weight
+    const void *b_rows;    // B rows slab of the pool
+    const float *v;        // [ksplit, T, MAX_RANK] shrink partials (read by the scaled reduce)
+    uint16_t *vhi;         // [T, MAX_RANK] hi part of scaling * intermediate
+    uint16_t *vlo;         // [T, MAX_RANK] lo part
+    int hin, hout;
+    int ksplit;
+    int ntn;               // column tiles (set by the launcher)
+    unsigned end;          // first workgroup id after this projection (set by the launcher)
+};
+
+struct GemmLoraArgs {
+    GemmProj pr[MAX_PROJ];
+    int n_proj;
+    int T;
+    int ntm;               // row tiles (set by the launcher)
+    int lora;              // 0: base product only
+    int rmax;              // rank columns the intermediate holds (16, 32 or 64; set by the launcher)
+    const int32_t *tile_rec;   // prefill plan records
+    const int32_t *n_tiles;    // [1]
+    int max_tiles;
+    long long n_rows_b;
+};
+
 // launchers (defined next to their kernels); return hipError_t as int
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);
@@ -147,6 +175,8 @@ int launch_assist_export(const AssistArgs &a, hipStream_t s);
 int launch_assist_import(const AssistArgs &a, hipStream_t s);
 constexpr int SGMV_PLAN = 1;    // write the tile list and records into the workspace
 constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already holds the plan unless SGMV_PLAN is set too)
+constexpr int SGMV_SHRINK = 4;  // the shrink launch alone: its partial sums feed the base GEMM + LoRA kernel
 int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s);
+int launch_gemm_lora(const GemmLoraArgs &a, int dtype, int max_rank, hipStream_t s);
 
 }  // namespace mlora

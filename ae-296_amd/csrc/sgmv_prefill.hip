@@ -536,7 +536,7 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
         rc = (int)hipGetLastError();
         if (rc) return rc;
     }
-    if (!(phases & SGMV_APPLY)) return 0;
+    if (!(phases & (SGMV_APPLY | SGMV_SHRINK))) return 0;
     // The caller has filled pr[], the shrink groups, ksplit, cols and ncb; the grid ends are set here.
     SgmvArgs g = a;
     unsigned end = 0;
@@ -553,7 +553,7 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
     const unsigned egrid = end;
     hipLaunchKernelGGL((sgmv_shrink_kernel<DT, RMAX>), dim3(sgrid), dim3(SG_NT), 0, s, g);
     rc = (int)hipGetLastError();
-    if (rc) return rc;
+    if (rc || !(phases & SGMV_APPLY)) return rc;
     {
         const long long n = (long long)g.T * (RMAX / 8);
         hipLaunchKernelGGL((sgmv_reduce_kernel<DT, RMAX>), dim3((unsigned)((n + 255) / 256), (unsigned)g.n_proj), dim3(256), 0, s, g);

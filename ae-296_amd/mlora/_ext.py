@@ -58,6 +58,8 @@ SIGNATURES = {
     "mlora_sgmv_multi_workspace_bytes": (_i64, [_i32, _i32, _i32]),
     "mlora_sgmv_multi_planned": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32,
                                         _i32, _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
+    "mlora_gemm_lora_planned": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32,
+                                       _i32, _i32, _i64, _i32, _i32, _vp, _i64, _vp]),
     "mlora_prefill_reflayout": (_i32, [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _vp]),
 }
 

@@ -318,6 +318,48 @@ def sgmv_multi(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: Ada
     _ext.check(rc)
 
 
+def gemm_lora(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], ws: Sequence[torch.Tensor], pool: Optional[AdapterPool],
+              layer: int, projs: Sequence[str], plan: Optional[PrefillPlan]) -> None:
+    """Base projection and LoRA in one pass for up to 8 projections of one prefill layer:
+    ``ys[p] = xs[p] @ ws[p] + delta`` with ``ws[p]`` the base weight as ``[hin, hout]`` (the layout of
+    ``layer_weight.q_weight_``), i.e. ``q = torch.mm(x, Wq); q += q_lora`` of
+    ``transformer_layer_infer.py:145-147,160-171`` with q written once.  ``plan=None`` (then ``pool`` may be
+    None and ``projs`` only names the outputs) runs the base products alone."""
+    n = len(projs)
+    if not (len(ys) == len(xs) == len(ws) == n) or not 1 <= n <= _ext.MAX_PROJ:
+        raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y, one x and one w each")
+    _need_cuda(*ys, *xs, *ws)
+    _need_contig(*ys, *xs, *ws)
+    T = xs[0].shape[0]
+    if plan is not None and plan.T != T:
+        raise ValueError("plan was built for a different number of tokens")
+    yv, xv, wv, av, bv, hi, ho = _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
+    dtype = xs[0].dtype
+    for i, p in enumerate(projs):
+        hin, hout = ws[i].shape
+        if plan is not None and tuple(pool.projections[p]) != (hin, hout):
+            raise ValueError(f"projection {p}: base weight is {tuple(ws[i].shape)}, the pool has {pool.projections[p]}")
+        if not (xs[i].dtype == ys[i].dtype == ws[i].dtype == dtype) or (plan is not None and dtype != pool.dtype):
+            raise TypeError("x, y, w and the pool must share one 16-bit dtype")
+        if tuple(xs[i].shape) != (T, hin) or tuple(ys[i].shape) != (T, hout):
+            raise ValueError(f"projection {p}: expected x [{T}, {hin}] and y [{T}, {hout}]")
+        yv[i], xv[i], wv[i], hi[i], ho[i] = ys[i].data_ptr(), xs[i].data_ptr(), ws[i].data_ptr(), hin, hout
+        if plan is not None:
+            av[i], bv[i] = pool.slab_ptrs(layer, p)
+    if plan is None:
+        rc = _ext.lib().mlora_gemm_lora_planned(n, yv, xv, wv, None, None, hi, ho, None, None, None, 0, None, None, None, T,
+                                                0, 0, 0, 0, 16, _ext.dtype_code(dtype), None, 0, _ext.current_stream_ptr())
+    else:
+        n_seg = _check_segments(plan.seg_start, plan.seg_len, plan.seg_adapter)
+        pool.sync()
+        rc = _ext.lib().mlora_gemm_lora_planned(
+            n, yv, xv, wv, av, bv, hi, ho, plan.seg_start.data_ptr(), plan.seg_len.data_ptr(), plan.seg_adapter.data_ptr(),
+            n_seg, _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling), T, pool.n_slots, pool.max_pages,
+            pool.page_rows, pool.n_pages, pool.max_rank, pool.dtype_code,
+            plan.workspace.data_ptr(), plan.workspace.numel(), _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
 def lora_prefill_ref(x: torch.Tensor, A_T: torch.Tensor, B_T: torch.Tensor, layer_idx: int,
                      workspace: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The reference's prefill expression on its own layout (``lora_gpu.py:125-128``):

@@ -256,6 +256,29 @@ int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x,
                              int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Base projection and LoRA in one pass, for the projections of one prefill layer:
+ *     y[p][t, :] = round16( x[p][t, :] . w[p]  +  scaling[a] * (x[p][t, :] . A_{p,a}) . B_{p,a} ),  a = adapter of t's segment
+ * with w[p] the base weight as [hin[p], hout[p]] row-major (the transposed layout lightllm keeps its
+ * projection weights in, layer_weights/transformer_layer_weight.py:44-46) and tokens outside every segment,
+ * or in a segment without adapter, getting the base product alone.  Replaces torch.mm(x, W) followed by
+ * `q += q_lora` (layer_infer/transformer_layer_infer.py:145-147 and :160-171), for which the reference
+ * writes y, reads it back and writes it again: here y is written once.  Launches: the SGMV shrink, a scaled
+ * reduce, and one GEMM launch for all projections in which the expand rides along as rank / 16 extra MFMA
+ * steps per output tile.  The sum is rounded to 16 bits once (the reference rounds the base product, the
+ * delta and their sum).  Arrays are HOST arrays of n_proj entries as in mlora_sgmv_multi_planned; the
+ * workspace must hold mlora_sgmv_multi_workspace_bytes(T, n_seg, n_proj) bytes and a plan written by
+ * mlora_sgmv_plan for these segments.  n_seg = 0 runs the base products alone (workspace and pool may be
+ * NULL).  Limits: every w[p] smaller than 4 GiB.
+ */
+int mlora_gemm_lora_planned(int n_proj, void *const *y, const void *const *x, const void *const *w,
+                            const void *const *a_rows, const void *const *b_rows,
+                            const int32_t *hin, const int32_t *hout,
+                            const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                            const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                            int T, int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                            int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * The reference's prefill call on its own layout (lora_gpu.py:125-128): request b uses
  * adapter slot b; x [B, Lpad, hin]; A_T [>=B, L, r, hin]; B_T [>=B, L, hout, r];
  * y [B, Lpad, hout] = (x[b] . A_T[b, layer]^T) . B_T[b, layer]^T   (y is overwritten).

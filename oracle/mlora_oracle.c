@@ -21,6 +21,7 @@
  *   orc_pool_gather, orc_build_segments, orc_build_chunks, orc_build_work, orc_sgmv_plan : vs numpy closed forms / enumeration
  *   orc_pool_scatter          : numpy fancy-index assignment
  *   orc_lora_apply_paged      : brute-force fp64 loops, one-hot, scale 0, library matmul
+ *   orc_gemm_lora_paged       : numpy matmul (fp64) of base product plus delta, integer-valued exact case, both rounding contracts
  *   orc_add_lora_bgmv_ref     : same expression through numpy on the reference layout
  *   orc_prefill_bmm_ref       : numpy matmul pairs (the reference's bmm.bmm)
  *   orc_cpu_lora_worker       : numpy fp32 matmul of the reference's one-line arithmetic
@@ -370,6 +371,90 @@ int orc_lora_apply_paged(uint16_t *y, const uint16_t *y0, const uint16_t *x,
         }
     }
     free(vd); free(vf);
+    return ORC_OK;
+}
+
+/* Base projection plus LoRA delta (lightllm/models/llama/layer_infer/transformer_layer_infer.py:145-147 then
+ * :160-171, with q_weight_ stored as [Hin, Hout], layer_weights/transformer_layer_weight.py:44-46):
+ *     q = torch.mm(x, Wq);  q += q_lora
+ * ref_rounding = 1 restates the reference's three roundings (mm result to 16 bits, delta to 16 bits, their
+ * sum to 16 bits); ref_rounding = 0 is this build's contract: base product and delta summed in fp32 and
+ * rounded once.  Accumulation in fp32 (acc64 = 0, ascending k) or fp64 (acc64 = 1).  Tokens with a negative
+ * adapter get the base product alone. */
+int orc_gemm_lora_paged(uint16_t *y, const uint16_t *x, const uint16_t *w,
+                        const uint16_t *a_rows, const uint16_t *b_rows, const int32_t *tok_adapter,
+                        const int32_t *a_page_tbl, const int32_t *b_page_tbl, const int32_t *rank, const float *scaling,
+                        int T, int Hin, int Hout, int n_adapters, int max_pages, int page_rows,
+                        int dtype, int acc64, int ref_rounding)
+{
+    if (T < 0 || Hin <= 0 || Hout <= 0 || max_pages <= 0 || page_rows <= 0) return ORC_EINVAL;
+    if (dtype != 0 && dtype != 1) return ORC_EINVAL;
+    for (int t = 0; t < T; t++) {
+        int a = tok_adapter[t];
+        if (a >= n_adapters) return ORC_ERANGE;
+        if (a >= 0 && (rank[a] + page_rows - 1) / page_rows > max_pages) return ORC_ERANGE;
+    }
+    double *base = (double *)malloc(sizeof(double) * (size_t)Hout);
+    float *basef = (float *)malloc(sizeof(float) * (size_t)Hout);
+    double *v = (double *)malloc(sizeof(double) * (size_t)max_pages * page_rows);
+    if (!base || !basef || !v) { free(base); free(basef); free(v); return ORC_EINVAL; }
+    for (int t = 0; t < T; t++) {
+        const uint16_t *xt = x + (size_t)t * Hin;
+        for (int c = 0; c < Hout; c++) { base[c] = 0.0; basef[c] = 0.0f; }
+        for (int k = 0; k < Hin; k++) {
+            const float xv = ld16(xt, k, dtype);
+            const uint16_t *wr = w + (size_t)k * Hout;
+            if (acc64) for (int c = 0; c < Hout; c++) base[c] += (double)xv * (double)ld16(wr, c, dtype);
+            else for (int c = 0; c < Hout; c++) basef[c] += xv * ld16(wr, c, dtype);
+        }
+        if (!acc64) for (int c = 0; c < Hout; c++) base[c] = basef[c];
+        int a = tok_adapter[t];
+        int r = a >= 0 ? rank[a] : 0;
+        for (int j = 0; j < r; j++) {
+            size_t row = (size_t)a_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+            const uint16_t *ar = a_rows + row * Hin;
+            if (acc64) {
+                double acc = 0.0;
+                for (int k = 0; k < Hin; k++) acc += (double)ld16(xt, k, dtype) * (double)ld16(ar, k, dtype);
+                v[j] = acc;
+            } else {
+                float acc = 0.0f;
+                for (int k = 0; k < Hin; k++) acc += ld16(xt, k, dtype) * ld16(ar, k, dtype);
+                v[j] = acc;
+            }
+        }
+        for (int c = 0; c < Hout; c++) {
+            double d = 0.0;
+            if (acc64) {
+                for (int j = 0; j < r; j++) {
+                    size_t row = (size_t)b_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+                    d += v[j] * (double)ld16(b_rows + row * Hout, c, dtype);
+                }
+                if (a >= 0) d *= (double)scaling[a];
+            } else {
+                float acc = 0.0f;
+                for (int j = 0; j < r; j++) {
+                    size_t row = (size_t)b_page_tbl[(size_t)a * max_pages + j / page_rows] * page_rows + j % page_rows;
+                    acc += (float)v[j] * ld16(b_rows + row * Hout, c, dtype);
+                }
+                d = a >= 0 ? (double)(scaling[a] * acc) : 0.0;
+            }
+            uint16_t out;
+            if (ref_rounding) {
+                uint16_t q = st16((float)base[c], dtype);
+                if (a >= 0) {
+                    uint16_t ql = st16((float)d, dtype);
+                    uint16_t one = q;
+                    q = st16(ld16(&one, 0, dtype) + ld16(&ql, 0, dtype), dtype);
+                }
+                out = q;
+            } else {
+                out = acc64 ? st16((float)(base[c] + d), dtype) : st16((float)base[c] + (float)d, dtype);
+            }
+            y[(size_t)t * Hout + c] = out;
+        }
+    }
+    free(base); free(basef); free(v);
     return ORC_OK;
 }
 

@@ -199,6 +199,30 @@ def lora_apply_paged(x, a_rows, b_rows, tok_adapter, a_page_tbl, b_page_tbl, ran
     return y
 
 
+def gemm_lora_paged(x, w, a_rows, b_rows, tok_adapter, a_page_tbl, b_page_tbl, rank, scaling, page_rows, dtype,
+                    acc64=False, ref_rounding=False):
+    """y = round16(x W + s_a (x A_a) B_a) (or the reference's three roundings); 16-bit arrays as uint16 bits."""
+    x = np.ascontiguousarray(x, np.uint16)
+    w = np.ascontiguousarray(w, np.uint16)
+    a_rows = np.ascontiguousarray(a_rows, np.uint16)
+    b_rows = np.ascontiguousarray(b_rows, np.uint16)
+    tok_adapter = np.ascontiguousarray(tok_adapter, np.int32)
+    a_page_tbl = np.ascontiguousarray(a_page_tbl, np.int32)
+    b_page_tbl = np.ascontiguousarray(b_page_tbl, np.int32)
+    rank = np.ascontiguousarray(rank, np.int32)
+    scaling = np.ascontiguousarray(scaling, np.float32)
+    T, Hin = x.shape
+    Hout = w.shape[1]
+    assert w.shape[0] == Hin and a_rows.shape[1] == Hin and b_rows.shape[1] == Hout
+    N, max_pages = a_page_tbl.shape
+    y = np.empty((T, Hout), np.uint16)
+    rc = lib().orc_gemm_lora_paged(_p(y), _p(x), _p(w), _p(a_rows), _p(b_rows), _p(tok_adapter), _p(a_page_tbl),
+                                   _p(b_page_tbl), _p(rank), _p(scaling), T, Hin, Hout, N, max_pages, page_rows,
+                                   dtype, int(acc64), int(ref_rounding))
+    _check(rc, "gemm_lora_paged")
+    return y
+
+
 def add_lora_bgmv_ref(y, x, wa_T_all, wb_T_all, indices, layer_idx, scale, dtype=FP16):
     """In place y += scale * x @ wa[idx, layer].T @ wb[idx, layer].T on the reference layout."""
     assert y.dtype == np.uint16 and y.flags["C_CONTIGUOUS"]

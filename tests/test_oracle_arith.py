@@ -239,3 +239,73 @@ def test_cpu_pool_equals_batch_over_many_wakeups():
                                   orc.cpu_lora_batch(x, down, up, req_adapter, tkn, cap, 2))
     finally:
         pool.close()
+
+
+# ---------------------------------------------------------------- base projection + LoRA (one pass)
+def _gemm_lora(pool, x_bits, w_bits, tok, **kw):
+    return orc.gemm_lora_paged(x_bits, w_bits, pool.a_rows, pool.b_rows, tok, pool.page_tbl, pool.page_tbl, pool.ranks,
+                               pool.scaling, pool.page_rows, pool.dtype, **kw)
+
+
+@pytest.mark.parametrize("dtype", [FP16, BF16])
+def test_gemm_lora_integer_inputs_bit_exact(dtype):
+    """Integer-valued operands: base product, delta and their sum are exact in fp32 and representable, so the
+    single-rounding contract, the reference's three roundings and numpy's integer matmul must all agree."""
+    rng = np.random.default_rng(70)
+    ranks = [8, 3, 16, 1]
+    pool = PagedPool(rng, ranks, hin=48, hout=40, page_rows=4, dtype=dtype, integer=True)
+    pool.scaling[:] = [1, 2, 0.5, -1]
+    T = 21
+    tok = rng.integers(-1, len(ranks), T).astype(np.int32)
+    xi = rng.integers(-2, 3, (T, 48)) * (rng.random((T, 48)) < 0.3)
+    wi = rng.integers(-1, 2, (48, 40))
+    want = (xi @ wi).astype(np.float64)
+    for t in range(T):
+        if tok[t] >= 0:
+            a = int(tok[t])
+            want[t] += pool.scaling[a] * (xi[t].astype(np.float64) @ pool.A(a) @ pool.B(a))
+    assert np.abs(want).max() < (2048 if dtype == FP16 else 256)
+    xb, wb = bits_of(xi.astype(np.float32), dtype), bits_of(wi.astype(np.float32), dtype)
+    for kw in (dict(), dict(acc64=True), dict(ref_rounding=True), dict(acc64=True, ref_rounding=True)):
+        assert np.array_equal(f32_of(_gemm_lora(pool, xb, wb, tok, **kw), dtype).astype(np.float64), want), kw
+
+
+@pytest.mark.parametrize("dtype", [FP16, BF16])
+def test_gemm_lora_is_library_matmul_plus_delta(dtype):
+    rng = np.random.default_rng(71)
+    pool = PagedPool(rng, [16, 8, 24], hin=256, hout=96, dtype=dtype)
+    T = 17
+    tok = rng.integers(-1, 3, T).astype(np.int32)
+    x = bits_of(rng.standard_normal((T, 256)).astype(np.float32), dtype)
+    w = bits_of((rng.standard_normal((256, 96)) * 0.05).astype(np.float32), dtype)
+    xf, wf = f32_of(x, dtype).astype(np.float64), f32_of(w, dtype).astype(np.float64)
+    want = xf @ wf
+    for t in range(T):
+        if tok[t] >= 0:
+            a = int(tok[t])
+            want[t] += pool.scaling[a] * (xf[t] @ pool.A(a) @ pool.B(a))
+    got64 = f32_of(_gemm_lora(pool, x, w, tok, acc64=True), dtype).astype(np.float64)
+    assert np.all(np.abs(got64 - want) <= 0.51 * ulp16(want, dtype))            # fp64 sums, one rounding
+    got32 = f32_of(_gemm_lora(pool, x, w, tok), dtype).astype(np.float64)
+    assert np.all(np.abs(got32 - want) <= 1.01 * ulp16(want, dtype) + 1e-5)     # fp32 sums over 256 terms
+    # the reference's three roundings: half an ulp each of the base product, the delta and their sum
+    got_ref = f32_of(_gemm_lora(pool, x, w, tok, ref_rounding=True, acc64=True), dtype).astype(np.float64)
+    base, delta = xf @ wf, want - xf @ wf
+    bound = 0.51 * (ulp16(base, dtype) + ulp16(delta, dtype) + ulp16(want, dtype)) + 0.51 * ulp16(got_ref, dtype)
+    assert np.all(np.abs(got_ref - want) <= bound)
+    assert np.any(got_ref != got64)                                              # and they do differ from one rounding
+    # without adapters it is the plain product; the delta alone is what lora_apply_paged computes
+    none = np.full(T, -1, np.int32)
+    base = f32_of(_gemm_lora(pool, x, w, none, acc64=True), dtype).astype(np.float64)
+    assert np.all(np.abs(base - xf @ wf) <= 0.51 * ulp16(xf @ wf, dtype))
+
+
+def test_gemm_lora_zero_weight_equals_lora_apply():
+    """W = 0 leaves the delta: bit-identical to the LoRA-only oracle with y = delta."""
+    rng = np.random.default_rng(72)
+    pool = PagedPool(rng, [16, 5], hin=128, hout=64, dtype=FP16)
+    T = 11
+    tok = rng.integers(-1, 2, T).astype(np.int32)
+    x = bits_of(rng.standard_normal((T, 128)).astype(np.float32), FP16)
+    w0 = np.zeros((128, 64), np.uint16)
+    assert np.array_equal(_gemm_lora(pool, x, w0, tok), _apply(pool, x, tok, None))
