@@ -12,10 +12,10 @@
 // rank / 16 more MFMA steps with (intermediate, B rows of its adapter) as operands.
 //
 // One workgroup (256 threads, 2 x 2 wavefronts of 128 x 128 outputs each) computes a 256 x 256 tile of y
-// on v_mfma_f32_32x32x16_{f16,bf16}.  K advances 64 columns per step through two LDS stages: while the
-// MFMAs of step k run from one stage, the registers holding step k+1 are parked in the other and the
-// global loads of step k+2 are in flight.  x is K-contiguous, so its operand is a plain 16-byte LDS read;
-// W is N-contiguous and is read back with the transposing LDS read.
+// on v_mfma_f32_32x32x16_{f16,bf16}.  K advances 32 columns per step through a ring of four LDS stages
+// that global memory fills directly (buffer_load ... lds): while the MFMAs of step k run from one stage, the
+// loads of steps k+1 .. k+3 are in flight or landed.  x is K-contiguous, so its operand is a plain 16-byte
+// LDS read; W is N-contiguous and is read back with the transposing LDS read.
 #include "mlora_args.hpp"
 #include "mlora_dev.hpp"
 #include <type_traits>
@@ -24,9 +24,9 @@ namespace mlora {
 
 constexpr int GM = 256;                 // rows (tokens) per tile
 constexpr int GN = 256;                 // output columns per tile
-constexpr int GK = 64;                  // K columns per stage
+constexpr int GK = 32;                  // K columns per stage
+constexpr int NST = 4;                  // stages in flight (a ring)
 constexpr int G_NT = 256;
-constexpr int PB = GN * 2 + 64;         // LDS pitch of a parked B row (expand step): the 4 rows x 32 bytes of a transposing read fall on distinct banks
 constexpr int A_BYTES = GM * GK * 2;    // x tile of a stage, rows unpadded and chunk-swizzled
 constexpr int B_BYTES = GK * GN * 2;    // W tile of a stage, likewise
 constexpr int STAGE = A_BYTES + B_BYTES;
@@ -35,8 +35,8 @@ constexpr int GROUP_M = 4;              // row tiles that share W column tiles b
 typedef short gl_short4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) gl_short4 gl_lds_short4;
 
-static_assert(2 * STAGE <= 160 * 1024 - 4096, "two stages and the small tables must fit the LDS of a compute unit");
-static_assert(4 * 32 * OPITCH <= STAGE && MAX_RANK * PB <= STAGE, "output staging and the parked B rows reuse a stage");
+static_assert(NST * STAGE <= 160 * 1024 - 4096, "the stages and the small tables must fit the LDS of a compute unit");
+static_assert(32 * OPITCH <= STAGE && MAX_RANK * GN * 2 <= STAGE, "a wavefront's output staging and the parked B rows each reuse one stage");
 
 template <int DT>
 __device__ __forceinline__ float16_t mfma32(const uint4 &a, const uint4 &b, float16_t c)
@@ -47,19 +47,10 @@ __device__ __forceinline__ float16_t mfma32(const uint4 &a, const uint4 &b, floa
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
 }
 
-// B operand of a 32x32x16 MFMA out of a row-major [k][n] LDS tile: lane (n = lane % 32, k group = lane / 32)
-// needs rows k0 + 8 * (lane / 32) + 0..7 of column n0 + lane % 32.  Each transposing read serves a 16-lane
-// group: lane i of the group addresses row i / 4, columns 4 * (i % 4) .. + 3, and receives the four rows of
-// column i.
-__device__ __forceinline__ uint4 lds_b_operand(const unsigned char *tile, int pitch, int k0, int n0, int lane)
-{
-    const int g = lane >> 4, m = lane & 15;
-    const unsigned char *src = tile + (k0 + 8 * (g >> 1) + (m >> 2)) * pitch + (n0 + (g & 1) * 16 + (m & 3) * 4) * 2;
-    const gl_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)src);
-    const gl_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)(src + 4 * pitch));
-    return make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
-                      __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
-}
+// The B operand of a 32x32x16 MFMA out of a row-major [k][n] LDS tile: lane (n = lane % 32, k group = lane / 32)
+// needs rows k0 + 8 * (lane / 32) + 0..7 of column n0 + lane % 32.  Each transposing read (ds_read_b64_tr_b16)
+// serves a 16-lane group: lane i of the group addresses row i / 4, columns 4 * (i % 4) .. + 3, and receives the
+// four rows of column i.
 
 // ------------------------------------------------------------------ scaled reduce
 // vhi + vlo [t][0..RMAX) = s_a * sum over the K splits of the shrink partials, for the tokens of one plan
@@ -104,9 +95,11 @@ __global__ __launch_bounds__(256) void gemm_lora_reduce_kernel(const GemmLoraArg
 template <int DT>
 __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p)
 {
-    // two stages as two arrays: the compiler then knows that parking step k + 1 cannot alias the operand reads of step k
+    // one array per stage: the compiler then knows that loads into one stage cannot alias the operand reads of another
     __shared__ __attribute__((aligned(16))) unsigned char smem[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char smem1[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char smem2[STAGE];
+    __shared__ __attribute__((aligned(16))) unsigned char smem3[STAGE];
     __shared__ unsigned long long s_mask[G_NT / 64];
 
     // ---- which projection, which tile.  Workgroups go to the 8 XCDs round-robin by id; every XCD works
@@ -126,7 +119,8 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     const int mt = grp * GROUP_M + within % rows_in_grp, nt = within / rows_in_grp;
     const int m0 = mt * GM, n0 = nt * GN;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // uniform, and the compiler may keep it in an SGPR
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
     const int T = p.T, hin = pj.hin, hout = pj.hout;
@@ -137,21 +131,21 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     // 64 lanes x 16 bytes into 1 KiB of consecutive LDS, lane i to slot i.  The tiles therefore have no row
     // padding; bank conflicts are avoided by storing 16-byte chunk c of a row at position c ^ key(row), which
     // costs nothing on the way in (lane i simply fetches the chunk that belongs in slot i).
-    //   x tile [256 rows][8 chunks]:  key = (row / 2) % 8   (16 operand rows of one chunk column -> 16 bank groups)
-    //   W tile [64 k rows][32 chunks]: key = (k % 4) * 4     (the 4 rows of a transposing read -> 4 bank groups)
-    // One load of wavefront w covers 8 rows of x (rows 8 (4 q + w) ..) or 2 rows of W (rows 2 (4 q + w) ..).
+    //   x tile [256 rows][4 chunks]:  key = (row / 4) % 4   (16 operand rows of one chunk column -> 16 bank groups)
+    //   W tile [32 k rows][32 chunks]: key = (k % 4) * 4     (the 4 rows of a transposing read -> 4 bank groups)
+    // One load of wavefront w covers 16 rows of x (rows 16 (4 q + w) ..) or 2 rows of W (rows 2 (4 q + w) ..).
     // Rows beyond T and columns beyond hout are clamped to valid addresses; what they produce is never stored.
     const int rows_here = T - m0 < GM ? T - m0 : GM;
-    unsigned aoff[8], boff[8];
+    unsigned aoff[4], boff[4];
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        const int row = 8 * (4 * q + wave) + (lane >> 3);
-        const int c = (lane & 7) ^ ((row >> 1) & 7);
+    for (int q = 0; q < 4; q++) {
+        const int row = 16 * (4 * q + wave) + (lane >> 2);
+        const int c = (lane & 3) ^ ((row >> 2) & 3);
         const int r = row < rows_here ? row : rows_here - 1;
         aoff[q] = ((unsigned)r * (unsigned)hin + (unsigned)c * 8u) * 2u;
     }
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
+    for (int q = 0; q < 4; q++) {
         const int k = 2 * (4 * q + wave) + (lane >> 5);
         const int c = (lane & 31) ^ ((k & 3) << 2);
         int col = n0 + c * 8;
@@ -166,18 +160,31 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
         const_cast<uint16_t *>(x + (size_t)m0 * hin), (short)0, (int)(x_bytes < 0xffffffffu ? x_bytes : 0xffffffffu), 0x00020000);
     const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<uint16_t *>(wgt), (short)0, (int)((size_t)hin * hout * 2), 0x00020000);
-    typedef __attribute__((address_space(3))) void lds_void;
-    auto dma_a = [&](unsigned char *stage, int kt) {
-        const unsigned soff = (unsigned)kt * (GK * 2);
-#pragma unroll
-        for (int q = 0; q < 8; q++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(xrs, (lds_void *)(stage + (4 * q + wave) * 1024), 16, (int)aoff[q], (int)soff, 0, 0);
+    // The loads are written as inline assembly: the compiler's own bookkeeping of loads that land in LDS waits
+    // for all of them before any LDS read that follows, which would serialise the ring; here the waits are
+    // explicit (GL_WAIT_LOADS below).  M0 carries the LDS address of the wavefront's 1 KiB chunk; nothing else
+    // in this kernel uses M0.
+    typedef int gl_i32x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) unsigned char lds_byte;
+    auto rsrc_words = [](const void *base, size_t bytes) {
+        const unsigned long long a = (unsigned long long)base;
+        const gl_i32x4 r = {(int)(unsigned)a, (int)((a >> 32) & 0xffffu), (int)(bytes < 0xffffffffu ? bytes : 0xffffffffu), 0x00020000};
+        return r;
     };
-    auto dma_b = [&](unsigned char *stage, int kt) {
-        const unsigned soff = (unsigned)kt * GK * (unsigned)hout * 2u;
+    const gl_i32x4 xrw = rsrc_words(x + (size_t)m0 * hin, x_bytes);
+    const gl_i32x4 wrw = rsrc_words(wgt, (size_t)hin * hout * 2);
+    auto dma1 = [](const gl_i32x4 &rs, unsigned lds_addr, unsigned voff, unsigned soff) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                     :: "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff));
+    };
+    // the 8 loads of one K step: 4 of x, 4 of W
+    auto dma = [&](unsigned char *stage, int ks) {
+        const unsigned soff_a = (unsigned)ks * (GK * 2), soff_b = (unsigned)ks * GK * (unsigned)hout * 2u;
+        const unsigned base = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)stage + (unsigned)wave * 1024u;
 #pragma unroll
-        for (int q = 0; q < 8; q++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(wrs, (lds_void *)(stage + A_BYTES + (4 * q + wave) * 1024), 16, (int)boff[q], (int)soff, 0, 0);
+        for (int q = 0; q < 4; q++) dma1(xrw, base + q * 4096, aoff[q], soff_a);
+#pragma unroll
+        for (int q = 0; q < 4; q++) dma1(wrw, base + A_BYTES + q * 4096, boff[q], soff_b);
     };
 
     float16_t acc[4][4];
@@ -191,33 +198,37 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     // Operand addresses inside a stage.  x: lane (row wm * 128 + 32 i + lane % 32, chunk 2 kk + lane / 32); the key
     // of the row does not depend on i.  W: lane group g = lane / 16, m = lane % 16 reads rows 16 kk + 8 (g / 2) +
     // m / 4 (+ 4), bytes of columns wn * 128 + 32 j + 16 (g % 2) + 4 (m % 4) ..; the key (m / 4) * 4 flips bits of j.
-    unsigned a_at[4], b_at[4];
+    unsigned a_at[2], b_at[4];
     {
-        const int row = wm * 128 + l32, key = (l32 >> 1) & 7;
+        const int row = wm * 128 + l32, key = (l32 >> 2) & 3;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) a_at[kk] = (unsigned)(row * (GK * 2) + (((2 * kk + lh) ^ key) << 4));
+        for (int kk = 0; kk < 2; kk++) a_at[kk] = (unsigned)(row * (GK * 2) + (((2 * kk + lh) ^ key) << 4));
         const int g = lane >> 4, m = lane & 15;
         const int krow = 8 * (g >> 1) + (m >> 2);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int c = wn * 16 + ((j ^ (m >> 2)) << 2) + (g & 1) * 2 + ((m & 3) >> 1);
-            b_at[j] = (unsigned)(A_BYTES + krow * (GN * 2) + c * 16 + (m & 1) * 8);
+            b_at[j] = (unsigned)(krow * (GN * 2) + c * 16 + (m & 1) * 8);
         }
     }
-    // Operands of one K = 16 step (4 x fragments, 4 W fragments), read one step ahead of the MFMAs that use them.
-    uint4 fa[2][4], fb[2][4];
-    auto frags = [&](const unsigned char *stage, auto kk_c, uint4 (&af)[4], uint4 (&bf)[4]) {
-        constexpr int kk = decltype(kk_c)::value;
-#pragma unroll
-        for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(stage + a_at[kk] + i * 32 * (GK * 2));
+    // W operands of one K = 16 slice out of a [k rows][512 bytes] swizzled tile at `tile`
+    auto w_frags = [&](const unsigned char *tile, int kk, uint4 (&bf)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const unsigned char *src = stage + b_at[j] + kk * 16 * (GN * 2);
+            const unsigned char *src = tile + b_at[j] + kk * 16 * (GN * 2);
             const gl_short4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)src);
             const gl_short4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)(src + 4 * (GN * 2)));
             bf[j] = make_uint4(__builtin_bit_cast(uint2, lo).x, __builtin_bit_cast(uint2, lo).y,
                                __builtin_bit_cast(uint2, hi).x, __builtin_bit_cast(uint2, hi).y);
         }
+    };
+    // Operands of one K = 16 slice (4 x fragments, 4 W fragments), read one slice ahead of the MFMAs that use them.
+    uint4 fa[2][4], fb[2][4];
+    auto frags = [&](const unsigned char *stage, auto kk_c, uint4 (&af)[4], uint4 (&bf)[4]) {
+        constexpr int kk = decltype(kk_c)::value;
+#pragma unroll
+        for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const uint4 *>(stage + a_at[kk] + i * 32 * (GK * 2));
+        w_frags(stage + A_BYTES, kk, bf);
     };
     auto mfma16x = [&](const uint4 (&af)[4], const uint4 (&bf)[4]) {
 #pragma unroll
@@ -227,8 +238,6 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     };
     using K0 = std::integral_constant<int, 0>;
     using K1 = std::integral_constant<int, 1>;
-    using K2 = std::integral_constant<int, 2>;
-    using K3 = std::integral_constant<int, 3>;
 #define GL_FENCE() __builtin_amdgcn_sched_barrier(0)
     // Scheduling hints: one MFMA, then at most one operand read and at most one global load, so that the memory
     // instructions issue in the shadow of the MFMAs instead of in a burst between them (an MFMA occupies its pipe
@@ -239,87 +248,116 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
         if (n_ < (n_ds_read)) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    \
         if (n_ < (n_load)) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);       \
     }
-    // One K step of 64 columns out of stage `cur`, four slices of 16.  Operand reads run one slice ahead of
-    // the MFMAs.  The barrier sits before the last slice: by then every wavefront has read all it needs from
-    // `cur` and the loads of step kt + 1 (requested a whole step earlier) have landed in the other stage, so the
-    // last slice's operand prefetch reads the other stage, and `cur` is free to receive step kt + 2 at once.
-    auto k_step = [&](auto cur_c, auto has1_c, auto has2_c, int kt) {
+    // s_waitcnt with only the vector-memory counter set: at most n loads of this wavefront still in flight
+    // (loads complete in order).
+#define GL_WAIT_LOADS(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+    // One K step of 32 columns out of stage `ks % 4`, two slices of 16.  Operand reads run one slice ahead of
+    // the MFMAs.  The barrier sits between the slices: by then every wavefront has read all it needs from this
+    // stage and its loads of step ks + 1 (requested three steps earlier) have landed, so the second slice's
+    // operand prefetch reads the next stage, and this stage is free to receive step ks + 4 at once.
+    // `steady`: steps ks + 1 .. ks + 4 all exist; otherwise the ends of the pipeline are checked.
+    auto k_step = [&](auto cur_c, auto steady_c, int ks, int ns) {
         constexpr int cur_i = decltype(cur_c)::value;
-        constexpr bool has1 = decltype(has1_c)::value, has2 = decltype(has2_c)::value;
-        unsigned char *cur = cur_i ? smem1 : smem, *nxt = cur_i ? smem : smem1;
+        constexpr bool steady = decltype(steady_c)::value;
+        unsigned char *cur = cur_i == 0 ? smem : cur_i == 1 ? smem1 : cur_i == 2 ? smem2 : smem3;
+        unsigned char *nxt = cur_i == 0 ? smem1 : cur_i == 1 ? smem2 : cur_i == 2 ? smem3 : smem;
         frags(cur, K1{}, fa[1], fb[1]);
         mfma16x(fa[0], fb[0]);
         GL_MIX(12, 0)
         GL_FENCE();
-        frags(cur, K2{}, fa[0], fb[0]);
-        mfma16x(fa[1], fb[1]);
-        GL_MIX(12, 0)
-        GL_FENCE();
-        frags(cur, K3{}, fa[1], fb[1]);
-        mfma16x(fa[0], fb[0]);
-        GL_MIX(12, 0)
-        GL_FENCE();
+        const bool more_loads = steady || ks + 4 < ns, more_steps = steady || ks + 1 < ns;
+        GL_WAIT_LOADS(steady ? 16 : 0);            // steady: the loads of steps ks + 2 and ks + 3 may still be in flight
         __syncthreads();
-        if constexpr (has2) { dma_a(cur, kt + 2); dma_b(cur, kt + 2); }
-        if constexpr (has1) frags(nxt, K0{}, fa[0], fb[0]);
-        mfma16x(fa[1], fb[1]);
-        GL_MIX(12, 16)
-        GL_FENCE();
+        // Second slice, scheduled by hand (the loads are assembly, which the scheduler will not interleave):
+        // after MFMA n comes operand read n of the next step's first slice (4 of x, then 8 halves of W) and,
+        // for n < 8, load n of step ks + 4 into the stage that has just been released.
+        const unsigned soff_a = (unsigned)(ks + 4) * (GK * 2), soff_b = (unsigned)(ks + 4) * GK * (unsigned)hout * 2u;
+        const unsigned lbase = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)cur + (unsigned)wave * 1024u;
+#pragma unroll
+        for (int n = 0; n < 16; n++) {
+            acc[n >> 2][n & 3] = mfma32<DT>(fa[1][n >> 2], fb[1][n & 3], acc[n >> 2][n & 3]);
+            if (more_steps) {
+                if (n < 4) {
+                    fa[0][n] = *reinterpret_cast<const uint4 *>(nxt + a_at[0] + n * 32 * (GK * 2));
+                } else if (n < 12) {
+                    const int j = (n - 4) >> 1;
+                    const unsigned char *src = nxt + A_BYTES + b_at[j] + ((n & 1) ? 4 * (GN * 2) : 0);
+                    const uint2 h = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((gl_lds_short4 *)src));
+                    if (n & 1) { fb[0][j].z = h.x; fb[0][j].w = h.y; } else { fb[0][j].x = h.x; fb[0][j].y = h.y; }
+                }
+            }
+            if (more_loads && n < 8) {
+                if (n < 4) dma1(xrw, lbase + n * 4096, aoff[n], soff_a);
+                else dma1(wrw, lbase + A_BYTES + (n - 4) * 4096, boff[n - 4], soff_b);
+            }
+            GL_FENCE();
+        }
     };
-    using St0 = std::integral_constant<int, 0>;
-    using St1 = std::integral_constant<int, 1>;
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
     using Yes = std::true_type;
     using No = std::false_type;
 
     // Full K steps run through the pipeline; a partial last step follows on its own.
-    const int nkf = hin / GK;
-    if (nkf > 0) {
-        dma_a(smem, 0);
-        dma_b(smem, 0);
-        if (nkf > 1) { dma_a(smem1, 1); dma_b(smem1, 1); }
+    const int ns = hin / GK;
+    if (ns > 0) {
+        dma(smem, 0);
+        if (ns > 1) dma(smem1, 1);
+        if (ns > 2) dma(smem2, 2);
+        if (ns > 3) dma(smem3, 3);
+        GL_WAIT_LOADS(0);
         __syncthreads();
         frags(smem, K0{}, fa[0], fb[0]);
-        int kt = 0;
+        int ks = 0;
 #pragma unroll 1
-        for (; kt + 4 <= nkf; kt += 2) {                                 // steady state; leaves 2 or 3 steps
-            k_step(St0{}, Yes{}, Yes{}, kt);
-            k_step(St1{}, Yes{}, Yes{}, kt + 1);
+        for (; ks + 8 <= ns; ks += 4) {                                  // all four steps have steps ks + 4 .. behind them
+            k_step(S0{}, Yes{}, ks, ns);
+            k_step(S1{}, Yes{}, ks + 1, ns);
+            k_step(S2{}, Yes{}, ks + 2, ns);
+            k_step(S3{}, Yes{}, ks + 3, ns);
         }
-        if (nkf - kt == 3) { k_step(St0{}, Yes{}, Yes{}, kt); k_step(St1{}, Yes{}, No{}, kt + 1); k_step(St0{}, No{}, No{}, kt + 2); }
-        else if (nkf - kt == 2) { k_step(St0{}, Yes{}, No{}, kt); k_step(St1{}, No{}, No{}, kt + 1); }
-        else k_step(St0{}, No{}, No{}, kt);
+#pragma unroll 1
+        for (; ks < ns; ks += 4) {                                       // the last (at most seven) steps
+            k_step(S0{}, No{}, ks, ns);
+            if (ks + 1 < ns) k_step(S1{}, No{}, ks + 1, ns);
+            if (ks + 2 < ns) k_step(S2{}, No{}, ks + 2, ns);
+            if (ks + 3 < ns) k_step(S3{}, No{}, ks + 3, ns);
+        }
     }
-    if (nkf * GK < hin) {
+    if (ns * GK < hin) {
         // Partial last K step: through registers, with chunks of x and rows of W beyond hin replaced by zeros,
-        // parked in the same swizzled layout.  Every wavefront has passed the last barrier of the pipeline.
+        // parked in the same swizzled layout.  Every wavefront has passed the last barrier of the pipeline and
+        // stage 1 is not being read (the last step read stage (ns - 1) % 4; use the one after it).
+        unsigned char *st = (ns & 3) == 0 ? smem : (ns & 3) == 1 ? smem1 : (ns & 3) == 2 ? smem2 : smem3;
         const int ncc = hin >> 3;
 #pragma unroll
-        for (int q = 0; q < 8; q++) {
-            const int row = 8 * (4 * q + wave) + (lane >> 3);
-            const int c = (lane & 7) ^ ((row >> 1) & 7);
-            const bool ok = nkf * 8 + c < ncc;
-            const unsigned back = ok ? 0u : (unsigned)(nkf * 8 + c - (ncc - 1)) * 16u;
-            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(aoff[q] - back), nkf * (GK * 2), 0);
-            *reinterpret_cast<uint4 *>(smem + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
+        for (int q = 0; q < 4; q++) {
+            const int row = 16 * (4 * q + wave) + (lane >> 2);
+            const int c = (lane & 3) ^ ((row >> 2) & 3);
+            const bool ok = ns * 4 + c < ncc;
+            const unsigned back = ok ? 0u : (unsigned)(ns * 4 + c - (ncc - 1)) * 16u;
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(xrs, (int)(aoff[q] - back), ns * (GK * 2), 0);
+            *reinterpret_cast<uint4 *>(st + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
         }
 #pragma unroll
-        for (int q = 0; q < 8; q++) {
-            const int k = nkf * GK + 2 * (4 * q + wave) + (lane >> 5);
+        for (int q = 0; q < 4; q++) {
+            const int k = ns * GK + 2 * (4 * q + wave) + (lane >> 5);
             const bool ok = k < hin;
             const unsigned back = ok ? 0u : (unsigned)(k - (hin - 1)) * (unsigned)hout * 2u;
-            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wrs, (int)(boff[q] - back), (int)((unsigned)nkf * GK * (unsigned)hout * 2u), 0);
-            *reinterpret_cast<uint4 *>(smem + A_BYTES + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
+            const u32x4_t v = __builtin_amdgcn_raw_buffer_load_b128(wrs, (int)(boff[q] - back), (int)((unsigned)ns * GK * (unsigned)hout * 2u), 0);
+            *reinterpret_cast<uint4 *>(st + A_BYTES + (4 * q + wave) * 1024 + lane * 16) = ok ? make_uint4(v.x, v.y, v.z, v.w) : zero16();
         }
         __syncthreads();
-        const int rem = hin - nkf * GK;
-        frags(smem, K0{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]);
-        if (rem > 16) { frags(smem, K1{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
-        if (rem > 32) { frags(smem, K2{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
-        if (rem > 48) { frags(smem, K3{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
-        __syncthreads();
+        const int rem = hin - ns * GK;
+        frags(st, K0{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]);
+        if (rem > 16) { frags(st, K1{}, fa[0], fb[0]); mfma16x(fa[0], fb[0]); }
     }
+    __syncthreads();                               // every wavefront is done with the stages
 #undef GL_FENCE
 #undef GL_MIX
+#undef GL_WAIT_LOADS
 
     // ---- LoRA expand as extra K columns.  Plan tiles (at most 64 consecutive tokens of one adapter) that
     // overlap this row block are found by scanning the tile list, 256 tiles at a time; for each, the B rows
@@ -328,7 +366,7 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     if (p.lora) {
         const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
         const int n_plan = p.n_tiles[0];
-        unsigned char *sb = smem;                  // [rank rows][PB]
+        unsigned char *sb = smem;                  // [rank rows][512 bytes], chunk-swizzled like a W tile
         for (int b0 = 0; b0 < n_plan; b0 += G_NT) {
             const int ti = b0 + tid;
             bool hit = false;
@@ -359,7 +397,7 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                         const int col = n0 + c * 8;
                         uint4 v = zero16();
                         if (row >= 0 && row < p.n_rows_b && col < hout) v = ldg16(brows + (size_t)row * hout + col);
-                        *reinterpret_cast<uint4 *>(sb + j * PB + c * 16) = v;
+                        *reinterpret_cast<uint4 *>(sb + j * (GN * 2) + ((c ^ ((j & 3) << 2)) << 4)) = v;
                     }
                     __syncthreads();
 #pragma unroll
@@ -373,11 +411,12 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                             uint4 vh = ldg16(pj.vhi + vrow + ks + 8 * lh);
                             uint4 vl = ldg16(pj.vlo + vrow + ks + 8 * lh);
                             if (!mine) { vh = zero16(); vl = zero16(); }
+                            uint4 bf[4];
+                            w_frags(sb, ks >> 4, bf);
 #pragma unroll
                             for (int j = 0; j < 4; j++) {
-                                const uint4 bf = lds_b_operand(sb, PB, ks, wn * 128 + j * 32, lane);
-                                acc[i][j] = mfma32<DT>(vh, bf, acc[i][j]);
-                                acc[i][j] = mfma32<DT>(vl, bf, acc[i][j]);
+                                acc[i][j] = mfma32<DT>(vh, bf[j], acc[i][j]);
+                                acc[i][j] = mfma32<DT>(vl, bf[j], acc[i][j]);
                             }
                         }
                     }
@@ -393,7 +432,7 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     // The tile is private to the wavefront and LDS operations of one wavefront complete in order, so no
     // barrier is needed; the accesses are volatile so that they stay in program order.
     {
-        unsigned char *so = smem + wave * (32 * OPITCH);
+        unsigned char *so = wave == 0 ? smem : wave == 1 ? smem1 : wave == 2 ? smem2 : smem3;
         typedef __attribute__((address_space(3))) volatile uint16_t lds_vu16;
         typedef __attribute__((address_space(3))) volatile u32x4_t lds_vu32x4;
         uint16_t *__restrict__ y = static_cast<uint16_t *>(pj.y);

@@ -28,6 +28,7 @@ for _p in (ROOT, os.path.join(ROOT, "ae-296_amd")):
         sys.path.insert(0, _p)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_BF16_TFLOPS = 2500.0      # dense bf16 / fp16 MFMA peak of the device
 # HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
 # profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
 # same runs).  Reported as roofline.traffic only when the run is that same configuration.
@@ -158,6 +159,84 @@ def bench_c4(args, dev):
                         "traffic": None if args.fused else MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
                                   "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
                         "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
+           "cpu_baseline": None}
+    print(json.dumps(out), flush=True)
+
+
+def bench_f1(args, dev):
+    """Base projection + LoRA in one pass on the config-4 batch (Llama-13B shapes, 16 requests U[128, 1024],
+    32 rank-64 adapters, bf16): one step = q, k, v, o, gate, up, down of one layer, y = x W + delta, as one
+    mlora_gemm_lora_planned call (shrink, scaled reduce, one GEMM launch).  The same step as the reference runs
+    it -- library GEMM per projection, then the SGMV kernels adding the delta -- is timed beside it."""
+    import numpy as np
+    import torch
+
+    import mlora
+    from mlora import workloads
+    rng = np.random.default_rng(1004)
+    lens = rng.integers(128, 1025, 16).astype(np.int32)
+    adapters = rng.integers(0, 32, 16).astype(np.int32)
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    T = int(lens.sum())
+    projections = workloads.LLAMA13B_ALL
+    pool = mlora.AdapterPool(1, projections, 32, 32 * 8, page_rows=8, max_rank=64, dtype=torch.bfloat16, device=dev)
+    workloads.fill_pool(pool, np.full(32, 64, np.int32), np.full(32, 0.5, np.float32), rng, seed=1004)
+    ss, sl, sa = (torch.from_numpy(a).to(dev) for a in (starts, lens, adapters))
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(4004)
+    x = {h: torch.randn(T, h, device=dev, generator=gen).bfloat16() for h in (5120, 13824)}
+    x_o = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
+    x_ffn = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
+    x_in = {"q": x[5120], "k": x[5120], "v": x[5120], "o": x_o, "gate": x_ffn, "up": x_ffn, "down": x[13824]}
+    names = list(projections)
+    w = {p: (torch.randn(projections[p], device=dev, generator=gen) / projections[p][0] ** 0.5).bfloat16() for p in names}
+    y = {p: torch.empty(T, projections[p][1], device=dev, dtype=torch.bfloat16) for p in names}
+    ws = mlora.sgmv_workspace(T, 16, dev, n_proj=len(names))
+
+    def fused():
+        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)
+        mlora.gemm_lora([y[p] for p in names], [x_in[p] for p in names], [w[p] for p in names], pool, 0, names, plan)
+
+    def unfused():
+        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)
+        for p in names:
+            torch.mm(x_in[p], w[p], out=y[p])
+        mlora.sgmv_multi([y[p] for p in names], [x_in[p] for p in names], pool, 0, names, plan)
+
+    def base_only():
+        for p in names:
+            torch.mm(x_in[p], w[p], out=y[p])
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms_unfused = timed(unfused)
+    ms_base = timed(base_only)
+    ms_per_step = timed(fused)
+    flops = sum(2.0 * T * hin * hout + 2.0 * 64 * (hin + hout) * T for hin, hout in projections.values())
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    out = {"metric": "base projection + LoRA prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
+           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "config-4 batch with base weights: Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
+                                  "32 rank-64 adapters, bf16; y = x W + delta in one pass", "tokens": T, "segments": 16,
+                      "library_gemm_then_sgmv_ms": ms_unfused, "library_gemm_alone_ms": ms_base,
+                      "speedup_over_library_gemm_then_sgmv": ms_unfused / ms_per_step},
+           "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                        "frac": tflops / MFMA_PEAK_BF16_TFLOPS, "traffic": None,
+                        "kernel": "sgmv shrink + scaled reduce + gemm_lora_kernel (one launch over the 7 projections)",
+                        "flops_per_step": flops},
            "cpu_baseline": None}
     print(json.dumps(out), flush=True)
 
@@ -318,11 +397,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap", "assist"],
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap", "assist", "f1"],
                     help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
                          "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB); "
                          "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters; "
-                         "swap = adapter swap-in from pinned host memory; assist = CPU-assist transport")
+                         "swap = adapter swap-in from pinned host memory; assist = CPU-assist transport; "
+                         "f1 = base projection + LoRA in one pass on the config-4 batch, with the library GEMM + SGMV sequence timed beside it")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -349,6 +429,8 @@ def main():
         del src, dst
     if args.workload == "c4":
         return bench_c4(args, dev)
+    if args.workload == "f1":
+        return bench_f1(args, dev)
     if args.workload == "swap":
         return bench_swap(args, dev)
     if args.workload == "assist":
