@@ -559,7 +559,11 @@ int mlora_gemm_lora_planned(int n_proj, void *const *y, const void *const *x, co
         if ((int64_t)256 * hin[p] * 2 >= (1LL << 32)) return fail(MLORA_ERANGE, "projection %d: hin too large", p);
         a.pr[p].y = y[p]; a.pr[p].x = x[p]; a.pr[p].hin = hin[p]; a.pr[p].hout = hout[p];
         g.pr[p].y = y[p]; g.pr[p].x = x[p]; g.pr[p].w = w[p]; g.pr[p].hin = hin[p]; g.pr[p].hout = hout[p];
-        if (lora) { a.pr[p].a_rows = a_rows[p]; a.pr[p].b_rows = b_rows[p]; g.pr[p].b_rows = b_rows[p]; }
+        if (lora) {
+            a.pr[p].a_rows = a_rows[p]; a.pr[p].b_rows = b_rows[p]; g.pr[p].b_rows = b_rows[p];
+            // the B rows slab is addressed through one descriptor as well
+            if ((int64_t)a.pool.n_rows_b * hout[p] * 2 >= 0xfff00000LL) return fail(MLORA_ERANGE, "projection %d: B rows slab of 4 GiB or more", p);
+        }
     }
     g.n_proj = n_proj; g.T = T; g.lora = lora ? 1 : 0;
     if (lora) {

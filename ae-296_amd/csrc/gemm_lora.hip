@@ -357,16 +357,85 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     __syncthreads();                               // every wavefront is done with the stages
 #undef GL_FENCE
 #undef GL_MIX
-#undef GL_WAIT_LOADS
 
     // ---- LoRA expand as extra K columns.  Plan tiles (at most 64 consecutive tokens of one adapter) that
-    // overlap this row block are found by scanning the tile list, 256 tiles at a time; for each, the B rows
-    // of its adapter for this column tile are parked in LDS and every 32-row block that overlaps the tile
-    // runs rank / 16 MFMA steps with the intermediate of the tile's rows (zero for the other rows).
+    // overlap this row block are found by scanning the tile list, 256 tiles at a time, and handled four at a
+    // time: the B rows of each tile's adapter for this column tile go straight into one of the four (now free)
+    // stages, in the W tile's layout; then every 32-row block runs, for each tile that overlaps it, rank / 16
+    // slices of two MFMAs per 32 columns with (hi, lo) of the intermediate of the tile's rows as the x operand
+    // (zero for the other rows).  The intermediate depends on the row only, so a block's operands are read
+    // once, one block ahead, whatever tiles cover it.
     if (p.lora) {
         const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
+        const size_t b_bytes = (size_t)p.n_rows_b * hout * 2;             // the launcher guarantees < 4 GiB
+        const gl_i32x4 brw = rsrc_words(brows, b_bytes);
         const int n_plan = p.n_tiles[0];
-        unsigned char *sb = smem;                  // [rank rows][512 bytes], chunk-swizzled like a W tile
+        const int kmax = p.rmax;
+        // (hi, lo) of rank columns 16 s + 8 (lane / 32) .. + 7 of this lane's row in 32-row block i
+        auto load_v = [&](int i, uint4 (&vh)[4], uint4 (&vl)[4]) {
+            int row = m0 + wm * 128 + i * 32 + l32;
+            row = row < T ? row : T - 1;
+            const size_t at = (size_t)row * MAX_RANK + 8 * lh;
+#pragma unroll
+            for (int sl = 0; sl < 4; sl++)
+                if (sl * 16 < kmax) { vh[sl] = ldg16(pj.vhi + at + sl * 16); vl[sl] = ldg16(pj.vlo + at + sl * 16); }
+        };
+        int run_tile[4], nrun = 0;
+        auto flush = [&]() {
+            // up to four tiles: request their B rows, then apply them
+            int kp[4], i0[4], i1[4];
+            __syncthreads();                       // the stages are free (main loop or previous batch done)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                if (q >= nrun) continue;
+                const int32_t *__restrict__ rec = p.tile_rec + (size_t)run_tile[q] * TILE_WORDS;
+                const int ntok = rec[0], r = rec[2] < kmax ? rec[2] : kmax, tok0 = rec[4];
+                kp[q] = (r + 15) & ~15;
+                i0[q] = tok0 - m0; i1[q] = tok0 + ntok - m0;              // rows of the block, may stick out on either side
+                unsigned char *stage = q == 0 ? smem : q == 1 ? smem1 : q == 2 ? smem2 : smem3;
+                const unsigned lbase = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)stage;
+                for (int jj = wave; jj * 2 < kp[q]; jj += 4) {            // one load = rank rows 2 jj and 2 jj + 1
+                    const int ra = rec[TILE_ROWS_AT + 2 * jj], rb = rec[TILE_ROWS_AT + 2 * jj + 1];
+                    const int j = 2 * jj + (lane >> 5);
+                    const int row = (lane >> 5) ? rb : ra;
+                    const int col = n0 + (((lane & 31) ^ ((j & 3) << 2)) << 3);
+                    // rows that do not exist and columns beyond hout read as zero: an offset outside the descriptor
+                    const unsigned voff = (row >= 0 && row < p.n_rows_b && col < hout)
+                                              ? ((unsigned)row * (unsigned)hout + (unsigned)col) * 2u : 0xfffffff0u;
+                    dma1(brw, lbase + jj * 1024, voff, 0u);
+                }
+            }
+            uint4 vh[2][4], vl[2][4];
+            load_v(0, vh[0], vl[0]);
+            GL_WAIT_LOADS(0);
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if (i + 1 < 4) load_v(i + 1, vh[(i + 1) & 1], vl[(i + 1) & 1]);
+                const int R0 = wm * 128 + i * 32, my = R0 + l32;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    if (q >= nrun || R0 + 32 <= i0[q] || R0 >= i1[q]) continue;       // uniform per wavefront
+                    const unsigned char *stage = q == 0 ? smem : q == 1 ? smem1 : q == 2 ? smem2 : smem3;
+                    const unsigned keep = (my >= i0[q] && my < i1[q]) ? 0xffffffffu : 0u;
+#pragma unroll
+                    for (int sl = 0; sl < 4; sl++) {
+                        if (sl * 16 >= kp[q]) continue;
+                        const uint4 h = vh[i & 1][sl], l = vl[i & 1][sl];
+                        const uint4 xh = make_uint4(h.x & keep, h.y & keep, h.z & keep, h.w & keep);
+                        const uint4 xl = make_uint4(l.x & keep, l.y & keep, l.z & keep, l.w & keep);
+                        uint4 bf[4];
+                        w_frags(stage, sl, bf);
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            acc[i][j] = mfma32<DT>(xh, bf[j], acc[i][j]);
+                            acc[i][j] = mfma32<DT>(xl, bf[j], acc[i][j]);
+                        }
+                    }
+                }
+            }
+            nrun = 0;
+        };
         for (int b0 = 0; b0 < n_plan; b0 += G_NT) {
             const int ti = b0 + tid;
             bool hit = false;
@@ -384,47 +453,17 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                 unsigned long long mask = s_mask[w4];
 #pragma unroll 1
                 while (mask) {
-                    const int cur = b0 + w4 * 64 + __builtin_ctzll(mask);
+                    const int t = b0 + w4 * 64 + __builtin_ctzll(mask);
                     mask &= mask - 1;
-                    const int32_t *__restrict__ rec = p.tile_rec + (size_t)cur * TILE_WORDS;
-                    const int ntok = rec[0], r = rec[2] < p.rmax ? rec[2] : p.rmax, tok0 = rec[4];
-                    const int kp = (r + 15) & ~15;
-                    const int i0 = tok0 - m0, i1 = tok0 + ntok - m0;      // rows of the block, may stick out on either side
-                    __syncthreads();               // the previous tile's B rows have been consumed
-                    for (int e = tid; e < kp * 32; e += G_NT) {
-                        const int j = e >> 5, c = e & 31;
-                        const int row = rec[TILE_ROWS_AT + j];
-                        const int col = n0 + c * 8;
-                        uint4 v = zero16();
-                        if (row >= 0 && row < p.n_rows_b && col < hout) v = ldg16(brows + (size_t)row * hout + col);
-                        *reinterpret_cast<uint4 *>(sb + j * (GN * 2) + ((c ^ ((j & 3) << 2)) << 4)) = v;
-                    }
-                    __syncthreads();
-#pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int R0 = wm * 128 + i * 32;
-                        if (R0 + 32 <= i0 || R0 >= i1) continue;          // uniform per wavefront
-                        const int my = R0 + l32;
-                        const bool mine = my >= i0 && my < i1;
-                        const size_t vrow = (size_t)(m0 + (mine ? my : i0 > 0 ? i0 : 0)) * MAX_RANK;
-                        for (int ks = 0; ks < kp; ks += 16) {
-                            uint4 vh = ldg16(pj.vhi + vrow + ks + 8 * lh);
-                            uint4 vl = ldg16(pj.vlo + vrow + ks + 8 * lh);
-                            if (!mine) { vh = zero16(); vl = zero16(); }
-                            uint4 bf[4];
-                            w_frags(sb, ks >> 4, bf);
-#pragma unroll
-                            for (int j = 0; j < 4; j++) {
-                                acc[i][j] = mfma32<DT>(vh, bf[j], acc[i][j]);
-                                acc[i][j] = mfma32<DT>(vl, bf[j], acc[i][j]);
-                            }
-                        }
-                    }
+                    if (nrun == 0) run_tile[0] = t; else if (nrun == 1) run_tile[1] = t; else if (nrun == 2) run_tile[2] = t; else run_tile[3] = t;
+                    if (++nrun == 4) flush();
                 }
             }
         }
+        if (nrun > 0) flush();
         __syncthreads();
     }
+#undef GL_WAIT_LOADS
 
     // ---- y: every wavefront passes its 128 x 128 block through a private LDS tile, 32 rows at a time, so
     // that the stores are 16 bytes wide and a 16-lane row covers 256 contiguous bytes of one token.
@@ -462,6 +501,12 @@ static int launch_gl(const GemmLoraArgs &a, hipStream_t s)
     GemmLoraArgs g = a;
     g.rmax = RMAX;
     g.ntm = (g.T + GM - 1) / GM;
+    // projections with the longest K loop first: their tiles take longest, and a long tile started last
+    // would leave the rest of the device idle at the end of the launch
+    for (int q = 1; q < g.n_proj; q++)
+        for (int r = q; r > 0 && g.pr[r].hin > g.pr[r - 1].hin; r--) {
+            const GemmProj t = g.pr[r]; g.pr[r] = g.pr[r - 1]; g.pr[r - 1] = t;
+        }
     unsigned end = 0;
     for (int q = 0; q < g.n_proj; q++) {
         g.pr[q].ntn = (g.pr[q].hout + GN - 1) / GN;

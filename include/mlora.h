@@ -268,7 +268,7 @@ int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x,
  * delta and their sum).  Arrays are HOST arrays of n_proj entries as in mlora_sgmv_multi_planned; the
  * workspace must hold mlora_sgmv_multi_workspace_bytes(T, n_seg, n_proj) bytes and a plan written by
  * mlora_sgmv_plan for these segments.  n_seg = 0 runs the base products alone (workspace and pool may be
- * NULL).  Limits: every w[p] smaller than 4 GiB.
+ * NULL).  Limits: every w[p] and every B rows slab smaller than 4 GiB.
  */
 int mlora_gemm_lora_planned(int n_proj, void *const *y, const void *const *x, const void *const *w,
                             const void *const *a_rows, const void *const *b_rows,
