@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void gemm_lora_reduce_kernel(const GemmLoraArg
 }
 
 // ------------------------------------------------------------------ GEMM + expand
-template <int DT>
+template <int DT, int RMAX>
 __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p)
 {
     // one array per stage: the compiler then knows that loads into one stage cannot alias the operand reads of another
@@ -124,6 +124,21 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
     const int T = p.T, hin = pj.hin, hout = pj.hout;
+
+    // Which plan tiles (at most 64 consecutive tokens of one adapter) overlap this row block: asked now, for the
+    // first 256 tiles of the plan, so that the answer is there when the K loop ends (one bit per tile).
+    auto tile_hits = [&](int ti, int n_plan) {
+        if (ti >= n_plan) return false;
+        const int32_t *rec = p.tile_rec + (size_t)ti * TILE_WORDS;
+        const int4 h = *reinterpret_cast<const int4 *>(rec);             // tokens, adapter, rank, scaling
+        const int tok0 = rec[4];
+        return h.y >= 0 && h.z > 0 && h.x > 0 && tok0 >= 0 && tok0 + h.x <= T && tok0 < m0 + GM && tok0 + h.x > m0;
+    };
+    const int n_plan = p.lora ? p.n_tiles[0] : 0;
+    if (p.lora) {
+        const unsigned long long bal = __ballot(tile_hits(tid, n_plan));
+        if (lane == 0) s_mask[wave] = bal;                                // visible after the first barrier below
+    }
     const uint16_t *__restrict__ x = static_cast<const uint16_t *>(pj.x);
     const uint16_t *__restrict__ wgt = static_cast<const uint16_t *>(pj.w);
 
@@ -369,43 +384,50 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
         const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
         const size_t b_bytes = (size_t)p.n_rows_b * hout * 2;             // the launcher guarantees < 4 GiB
         const gl_i32x4 brw = rsrc_words(brows, b_bytes);
-        const int n_plan = p.n_tiles[0];
-        const int kmax = p.rmax;
+        constexpr int NSL = RMAX / 16;             // rank rows an adapter does not have read as zeros on both sides,
+                                                   // so every tile runs the same RMAX / 16 slices
         // (hi, lo) of rank columns 16 s + 8 (lane / 32) .. + 7 of this lane's row in 32-row block i
-        auto load_v = [&](int i, uint4 (&vh)[4], uint4 (&vl)[4]) {
+        auto load_v = [&](int i, uint4 (&vh)[NSL], uint4 (&vl)[NSL]) {
             int row = m0 + wm * 128 + i * 32 + l32;
             row = row < T ? row : T - 1;
             const size_t at = (size_t)row * MAX_RANK + 8 * lh;
 #pragma unroll
-            for (int sl = 0; sl < 4; sl++)
-                if (sl * 16 < kmax) { vh[sl] = ldg16(pj.vhi + at + sl * 16); vl[sl] = ldg16(pj.vlo + at + sl * 16); }
+            for (int sl = 0; sl < NSL; sl++) { vh[sl] = ldg16(pj.vhi + at + sl * 16); vl[sl] = ldg16(pj.vlo + at + sl * 16); }
         };
         int run_tile[4], nrun = 0;
         auto flush = [&]() {
             // up to four tiles: request their B rows, then apply them
-            int kp[4], i0[4], i1[4];
+            int i0[4], i1[4];
             __syncthreads();                       // the stages are free (main loop or previous batch done)
+            // Row of every rank row this lane will fetch: one load covers rank rows 2 jj and 2 jj + 1 (lanes 0..31 and
+            // 32..63), jj = wave, wave + 4, ...  All of these small loads are issued before any of them is used.
+            constexpr int NLD = RMAX / 8;          // loads per wavefront and tile
+            int rowv[4][NLD];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int32_t *__restrict__ rec = p.tile_rec + (size_t)run_tile[q < nrun ? q : 0] * TILE_WORDS;
+                const int ntok = rec[0], tok0 = rec[4];
+                i0[q] = tok0 - m0; i1[q] = tok0 + ntok - m0;              // rows of the block, may stick out on either side
+#pragma unroll
+                for (int u = 0; u < NLD; u++) rowv[q][u] = rec[TILE_ROWS_AT + 2 * (wave + 4 * u) + (lane >> 5)];
+            }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 if (q >= nrun) continue;
-                const int32_t *__restrict__ rec = p.tile_rec + (size_t)run_tile[q] * TILE_WORDS;
-                const int ntok = rec[0], r = rec[2] < kmax ? rec[2] : kmax, tok0 = rec[4];
-                kp[q] = (r + 15) & ~15;
-                i0[q] = tok0 - m0; i1[q] = tok0 + ntok - m0;              // rows of the block, may stick out on either side
                 unsigned char *stage = q == 0 ? smem : q == 1 ? smem1 : q == 2 ? smem2 : smem3;
-                const unsigned lbase = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)stage;
-                for (int jj = wave; jj * 2 < kp[q]; jj += 4) {            // one load = rank rows 2 jj and 2 jj + 1
-                    const int ra = rec[TILE_ROWS_AT + 2 * jj], rb = rec[TILE_ROWS_AT + 2 * jj + 1];
-                    const int j = 2 * jj + (lane >> 5);
-                    const int row = (lane >> 5) ? rb : ra;
+                const unsigned lbase = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)stage + (unsigned)wave * 1024u;
+#pragma unroll
+                for (int u = 0; u < NLD; u++) {
+                    const int j = 2 * (wave + 4 * u) + (lane >> 5);
+                    const int row = rowv[q][u];
                     const int col = n0 + (((lane & 31) ^ ((j & 3) << 2)) << 3);
                     // rows that do not exist and columns beyond hout read as zero: an offset outside the descriptor
                     const unsigned voff = (row >= 0 && row < p.n_rows_b && col < hout)
                                               ? ((unsigned)row * (unsigned)hout + (unsigned)col) * 2u : 0xfffffff0u;
-                    dma1(brw, lbase + jj * 1024, voff, 0u);
+                    dma1(brw, lbase + u * 4096, voff, 0u);
                 }
             }
-            uint4 vh[2][4], vl[2][4];
+            uint4 vh[2][NSL], vl[2][NSL];
             load_v(0, vh[0], vl[0]);
             GL_WAIT_LOADS(0);
             __syncthreads();
@@ -418,18 +440,18 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                     if (q >= nrun || R0 + 32 <= i0[q] || R0 >= i1[q]) continue;       // uniform per wavefront
                     const unsigned char *stage = q == 0 ? smem : q == 1 ? smem1 : q == 2 ? smem2 : smem3;
                     const unsigned keep = (my >= i0[q] && my < i1[q]) ? 0xffffffffu : 0u;
+                    uint4 bf[2][4];                 // W-side operands, one slice ahead
+                    w_frags(stage, 0, bf[0]);
 #pragma unroll
-                    for (int sl = 0; sl < 4; sl++) {
-                        if (sl * 16 >= kp[q]) continue;
+                    for (int sl = 0; sl < NSL; sl++) {
+                        if (sl + 1 < NSL) w_frags(stage, sl + 1, bf[(sl + 1) & 1]);
                         const uint4 h = vh[i & 1][sl], l = vl[i & 1][sl];
                         const uint4 xh = make_uint4(h.x & keep, h.y & keep, h.z & keep, h.w & keep);
                         const uint4 xl = make_uint4(l.x & keep, l.y & keep, l.z & keep, l.w & keep);
-                        uint4 bf[4];
-                        w_frags(stage, sl, bf);
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
-                            acc[i][j] = mfma32<DT>(xh, bf[j], acc[i][j]);
-                            acc[i][j] = mfma32<DT>(xl, bf[j], acc[i][j]);
+                            acc[i][j] = mfma32<DT>(xh, bf[sl & 1][j], acc[i][j]);
+                            acc[i][j] = mfma32<DT>(xl, bf[sl & 1][j], acc[i][j]);
                         }
                     }
                 }
@@ -437,17 +459,12 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
             nrun = 0;
         };
         for (int b0 = 0; b0 < n_plan; b0 += G_NT) {
-            const int ti = b0 + tid;
-            bool hit = false;
-            if (ti < n_plan) {
-                const int32_t *rec = p.tile_rec + (size_t)ti * TILE_WORDS;
-                const int ntok = rec[0], tok0 = rec[4];
-                hit = rec[1] >= 0 && rec[2] > 0 && ntok > 0 && tok0 >= 0 && tok0 + ntok <= T && tok0 < m0 + GM && tok0 + ntok > m0;
+            if (b0 > 0) {                          // the first 256 tiles were looked at before the K loop
+                const unsigned long long bal = __ballot(tile_hits(b0 + tid, n_plan));
+                __syncthreads();                   // s_mask of the previous batch has been consumed
+                if (lane == 0) s_mask[wave] = bal;
+                __syncthreads();
             }
-            const unsigned long long bal = __ballot(hit);
-            __syncthreads();                       // s_mask of the previous batch has been consumed
-            if (lane == 0) s_mask[wave] = bal;
-            __syncthreads();
 #pragma unroll 1
             for (int w4 = 0; w4 < G_NT / 64; w4++) {
                 unsigned long long mask = s_mask[w4];
@@ -522,7 +539,7 @@ static int launch_gl(const GemmLoraArgs &a, hipStream_t s)
         const int rc = (int)hipGetLastError();
         if (rc) return rc;
     }
-    hipLaunchKernelGGL((gemm_lora_kernel<DT>), dim3(end), dim3(G_NT), 0, s, g);
+    hipLaunchKernelGGL((gemm_lora_kernel<DT, RMAX>), dim3(end), dim3(G_NT), 0, s, g);
     return (int)hipGetLastError();
 }
 
