@@ -365,7 +365,7 @@ struct SgmvWs { int max_tiles; int ksplit; size_t off_rec, off_proj, per_proj, o
 SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
 {
     SgmvWs w;
-    w.max_tiles = T / SG_TM + n_seg + 1;
+    w.max_tiles = T / SG_TM + 2 * n_seg + 1;       // aligned cuts can add one partial tile at either end of a segment
     // shrink workgroups: about three per CU for a single projection; a call over several projections
     // has that many already with fewer splits, and fewer splits mean less partial-sum traffic
     const long long per_split = (long long)w.max_tiles * n_proj;
@@ -435,7 +435,7 @@ static int sgmv_common(int n_proj, void *const *y, const void *const *x, const v
                        const int32_t *seg_len, const int32_t *seg_adapter, int n_seg, const int32_t *page_tbl,
                        const int32_t *rank, const float *scaling, int T, int n_adapters,
                        int max_pages, int page_rows, int64_t n_pages, int max_rank, int dtype, int accumulate,
-                       void *workspace, int64_t workspace_bytes, int phases, void *stream)
+                       void *workspace, int64_t workspace_bytes, int phases, void *stream, int tile_aligned = 0)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (T < 0 || n_seg < 0) return fail(MLORA_EINVAL, "T and n_seg must be >= 0 (got %d, %d)", T, n_seg);
@@ -466,7 +466,7 @@ static int sgmv_common(int n_proj, void *const *y, const void *const *x, const v
     if (workspace_bytes < (int64_t)w.total)
         return fail(MLORA_ENOSPACE, "workspace has %lld bytes, %lld needed", (long long)workspace_bytes, (long long)w.total);
     a.seg_start = seg_start; a.seg_len = seg_len; a.seg_adapter = seg_adapter; a.n_seg = n_seg;
-    a.T = T; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0;
+    a.T = T; a.accumulate = accumulate ? 1 : 0; a.b_transposed = 0; a.seg_uniform_len = 0; a.tile_aligned = tile_aligned;
     carve(a, workspace, w);
     rc = mlora::launch_sgmv(a, dtype, max_rank, phases, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "sgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
@@ -495,6 +495,16 @@ int mlora_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, const int3
     return sgmv_common(1, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, seg_start, seg_len, seg_adapter, n_seg,
                        page_tbl, rank, scaling, T, n_adapters, max_pages, page_rows, n_pages, max_rank, MLORA_F16, 0,
                        workspace, workspace_bytes, mlora::SGMV_PLAN, stream);
+}
+
+int mlora_sgmv_plan_aligned(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                            const int32_t *page_tbl, const int32_t *rank, const float *scaling, int T, int n_adapters,
+                            int max_pages, int page_rows, int64_t n_pages, int max_rank, void *workspace,
+                            int64_t workspace_bytes, void *stream)
+{
+    return sgmv_common(1, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, seg_start, seg_len, seg_adapter, n_seg,
+                       page_tbl, rank, scaling, T, n_adapters, max_pages, page_rows, n_pages, max_rank, MLORA_F16, 0,
+                       workspace, workspace_bytes, mlora::SGMV_PLAN, stream, 1);
 }
 
 int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *seg_start,

@@ -101,6 +101,9 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     __shared__ __attribute__((aligned(16))) unsigned char smem2[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char smem3[STAGE];
     __shared__ unsigned long long s_mask[G_NT / 64];
+    __shared__ int s_list[G_NT + 1];               // plan tiles (of the 256 looked at) that overlap this row block; [G_NT] = how many
+    __shared__ int s_rows[4][MAX_RANK];            // row of every rank row of the (up to four) plan tiles being applied
+    __shared__ int s_span[4][2];                   // their first and one-past-last row, relative to this row block
 
     // ---- which projection, which tile.  Workgroups go to the 8 XCDs round-robin by id; every XCD works
     // through one contiguous range of the tile order below, in which GROUP_M row tiles sweep the column
@@ -135,9 +138,31 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
         return h.y >= 0 && h.z > 0 && h.x > 0 && tok0 >= 0 && tok0 + h.x <= T && tok0 < m0 + GM && tok0 + h.x > m0;
     };
     const int n_plan = p.lora ? p.n_tiles[0] : 0;
+    // s_list = the tiles among plan tiles b0 .. b0 + 255 that overlap this row block, in order (two barriers inside)
+    auto list_tiles = [&](int b0) {
+        const bool hit = tile_hits(b0 + tid, n_plan);
+        const unsigned long long bal = __ballot(hit);
+        if (lane == 0) s_mask[wave] = bal;
+        __syncthreads();
+        int before = 0;
+        for (int w4 = 0; w4 < wave; w4++) before += __builtin_popcountll(s_mask[w4]);
+        if (hit) s_list[before + __builtin_popcountll(bal & ((1ull << lane) - 1))] = b0 + tid;
+        if (tid == G_NT - 1) s_list[G_NT] = before + __builtin_popcountll(bal);
+        __syncthreads();
+    };
+    // thread (q, j) = (tid / 64, tid % 64) copies rank row j's row index of tile s_list[base + q] into LDS
+    auto fill_rows = [&](int base, int count) {
+        const int q = tid >> 6, j = tid & 63;
+        if (base + q < count) {
+            const int32_t *rec = p.tile_rec + (size_t)s_list[base + q] * TILE_WORDS;
+            s_rows[q][j] = rec[TILE_ROWS_AT + j];
+            if (j < 2) s_span[q][j] = rec[4] - m0 + (j ? rec[0] : 0);
+        }
+    };
     if (p.lora) {
-        const unsigned long long bal = __ballot(tile_hits(tid, n_plan));
-        if (lane == 0) s_mask[wave] = bal;                                // visible after the first barrier below
+        // the first four overlapping tiles: their records are fetched now, behind the K loop
+        list_tiles(0);
+        fill_rows(0, s_list[G_NT]);                // visible after the barrier that opens the K loop
     }
     const uint16_t *__restrict__ x = static_cast<const uint16_t *>(pj.x);
     const uint16_t *__restrict__ wgt = static_cast<const uint16_t *>(pj.w);
@@ -271,6 +296,17 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     // stage and its loads of step ks + 1 (requested three steps earlier) have landed, so the second slice's
     // operand prefetch reads the next stage, and this stage is free to receive step ks + 4 at once.
     // `steady`: steps ks + 1 .. ks + 4 all exist; otherwise the ends of the pipeline are checked.
+    const gl_i32x4 brw = rsrc_words(pj.b_rows, (size_t)p.n_rows_b * hout * 2);   // the launcher guarantees < 4 GiB
+    // one load = rank rows 2 jj and 2 jj + 1 (lanes 0..31 and 32..63) of tile q, jj = wave + 4 u, row indices from s_rows
+    auto b_row_of = [&](int q, int u) { return s_rows[q][2 * (wave + 4 * u) + (lane >> 5)]; };
+    auto b_rows_load = [&](int row, int u, unsigned lds_stage_wave) {
+        const int j = 2 * (wave + 4 * u) + (lane >> 5);
+        const int col = n0 + (((lane & 31) ^ ((j & 3) << 2)) << 3);
+        // rows that do not exist and columns beyond hout read as zero: an offset outside the descriptor
+        const unsigned voff = (row >= 0 && row < p.n_rows_b && col < hout)
+                                  ? ((unsigned)row * (unsigned)hout + (unsigned)col) * 2u : 0xfffffff0u;
+        dma1(brw, lds_stage_wave + u * 4096, voff, 0u);
+    };
     auto k_step = [&](auto cur_c, auto steady_c, int ks, int ns) {
         constexpr int cur_i = decltype(cur_c)::value;
         constexpr bool steady = decltype(steady_c)::value;
@@ -373,17 +409,13 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
 #undef GL_FENCE
 #undef GL_MIX
 
-    // ---- LoRA expand as extra K columns.  Plan tiles (at most 64 consecutive tokens of one adapter) that
-    // overlap this row block are found by scanning the tile list, 256 tiles at a time, and handled four at a
-    // time: the B rows of each tile's adapter for this column tile go straight into one of the four (now free)
-    // stages, in the W tile's layout; then every 32-row block runs, for each tile that overlaps it, rank / 16
-    // slices of two MFMAs per 32 columns with (hi, lo) of the intermediate of the tile's rows as the x operand
-    // (zero for the other rows).  The intermediate depends on the row only, so a block's operands are read
-    // once, one block ahead, whatever tiles cover it.
+    // ---- LoRA expand as extra K columns.  The plan tiles that overlap this row block (listed in LDS, 256 plan
+    // tiles at a time) are handled four at a time: the B rows of each tile's adapter for this column tile go
+    // straight into one of the four (now free) stages, in the W tile's layout; then every 32-row block runs, for each tile that overlaps it, RMAX / 16 slices
+    // of two MFMAs per 32 columns with (hi, lo) of the intermediate of the tile's rows as the x operand (zero
+    // for the other rows).  The intermediate depends on the row only, so a block's operands are read once,
+    // one block ahead, whatever tiles cover it.
     if (p.lora) {
-        const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(pj.b_rows);
-        const size_t b_bytes = (size_t)p.n_rows_b * hout * 2;             // the launcher guarantees < 4 GiB
-        const gl_i32x4 brw = rsrc_words(brows, b_bytes);
         constexpr int NSL = RMAX / 16;             // rank rows an adapter does not have read as zeros on both sides,
                                                    // so every tile runs the same RMAX / 16 slices
         // (hi, lo) of rank columns 16 s + 8 (lane / 32) .. + 7 of this lane's row in 32-row block i
@@ -394,22 +426,18 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
 #pragma unroll
             for (int sl = 0; sl < NSL; sl++) { vh[sl] = ldg16(pj.vhi + at + sl * 16); vl[sl] = ldg16(pj.vlo + at + sl * 16); }
         };
-        int run_tile[4], nrun = 0;
-        auto flush = [&]() {
-            // up to four tiles: request their B rows, then apply them
+        // up to four tiles (s_list[base .. base + nrun)): request their B rows, then apply them
+        auto flush = [&](int base, int count, int nrun, bool first) {
             int i0[4], i1[4];
-            __syncthreads();                       // the stages are free (main loop or previous batch done)
-            // Row of every rank row this lane will fetch: one load covers rank rows 2 jj and 2 jj + 1 (lanes 0..31 and
-            // 32..63), jj = wave, wave + 4, ...  All of these small loads are issued before any of them is used.
-            constexpr int NLD = RMAX / 8;          // loads per wavefront and tile
-            int rowv[4][NLD];
+            __syncthreads();                       // the stages and the tables are free (main loop or previous batch done)
+            if (!first) {
+                fill_rows(base, count);
+                __syncthreads();
+            }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int32_t *__restrict__ rec = p.tile_rec + (size_t)run_tile[q < nrun ? q : 0] * TILE_WORDS;
-                const int ntok = rec[0], tok0 = rec[4];
-                i0[q] = tok0 - m0; i1[q] = tok0 + ntok - m0;              // rows of the block, may stick out on either side
-#pragma unroll
-                for (int u = 0; u < NLD; u++) rowv[q][u] = rec[TILE_ROWS_AT + 2 * (wave + 4 * u) + (lane >> 5)];
+                i0[q] = __builtin_amdgcn_readfirstlane(s_span[q][0]);    // rows of the block, may stick out on either side
+                i1[q] = __builtin_amdgcn_readfirstlane(s_span[q][1]);
             }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
@@ -417,15 +445,7 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                 unsigned char *stage = q == 0 ? smem : q == 1 ? smem1 : q == 2 ? smem2 : smem3;
                 const unsigned lbase = (unsigned)(__UINTPTR_TYPE__)(lds_byte *)stage + (unsigned)wave * 1024u;
 #pragma unroll
-                for (int u = 0; u < NLD; u++) {
-                    const int j = 2 * (wave + 4 * u) + (lane >> 5);
-                    const int row = rowv[q][u];
-                    const int col = n0 + (((lane & 31) ^ ((j & 3) << 2)) << 3);
-                    // rows that do not exist and columns beyond hout read as zero: an offset outside the descriptor
-                    const unsigned voff = (row >= 0 && row < p.n_rows_b && col < hout)
-                                              ? ((unsigned)row * (unsigned)hout + (unsigned)col) * 2u : 0xfffffff0u;
-                    dma1(brw, lbase + u * 4096, voff, 0u);
-                }
+                for (int u = 0; u < RMAX / 8; u++) b_rows_load(b_row_of(q, u), u, lbase);
             }
             uint4 vh[2][NSL], vl[2][NSL];
             load_v(0, vh[0], vl[0]);
@@ -456,28 +476,16 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
                     }
                 }
             }
-            nrun = 0;
         };
+#pragma unroll 1
         for (int b0 = 0; b0 < n_plan; b0 += G_NT) {
-            if (b0 > 0) {                          // the first 256 tiles were looked at before the K loop
-                const unsigned long long bal = __ballot(tile_hits(b0 + tid, n_plan));
-                __syncthreads();                   // s_mask of the previous batch has been consumed
-                if (lane == 0) s_mask[wave] = bal;
-                __syncthreads();
-            }
+            if (b0 > 0) list_tiles(b0);            // the first 256 tiles were looked at before the K loop
+            const int count = __builtin_amdgcn_readfirstlane(s_list[G_NT]);
 #pragma unroll 1
-            for (int w4 = 0; w4 < G_NT / 64; w4++) {
-                unsigned long long mask = s_mask[w4];
-#pragma unroll 1
-                while (mask) {
-                    const int t = b0 + w4 * 64 + __builtin_ctzll(mask);
-                    mask &= mask - 1;
-                    if (nrun == 0) run_tile[0] = t; else if (nrun == 1) run_tile[1] = t; else if (nrun == 2) run_tile[2] = t; else run_tile[3] = t;
-                    if (++nrun == 4) flush();
-                }
-            }
+            for (int base = 0; base < count; base += 4)
+                flush(base, count, count - base < 4 ? count - base : 4, b0 == 0 && base == 0);
+            __syncthreads();                       // s_list is free for the next 256 tiles
         }
-        if (nrun > 0) flush();
         __syncthreads();
     }
 #undef GL_WAIT_LOADS

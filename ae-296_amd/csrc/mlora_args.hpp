@@ -127,6 +127,7 @@ struct SgmvArgs {
     int accumulate;
     int b_transposed;      // B given as [hout, r] blocks (reference layout)
     int seg_uniform_len;   // > 0: segment s covers [s*len, (s+1)*len), adapter s (reference prefill)
+    int tile_aligned;      // plan: cut tiles at multiples of 64 tokens (and at segment ends) instead of every 64 tokens of a segment
     // workspace carve-up
     int32_t *tile_seg;     // [max_tiles]
     int32_t *tile_tok0;

@@ -1,7 +1,7 @@
 // SGMV prefill kernels for gfx950: tokens are packed per segment (one adapter per segment)
 //     y[t] (+)= s_a * (x[t] . A_a) . B_a
 // computed on v_mfma_f32_16x16x32_{f16,bf16} tiles in four launches on one stream (the first can be shared by all projections and layers of a batch):
-//   plan   : cuts every segment into tiles of 64 tokens (work list in the workspace);
+//   plan   : cuts every segment into tiles of at most 64 tokens (work list in the workspace);
 //   shrink : V[split][t][0..R) = x[t, Kslice] . A_a[:, Kslice]^T   (split-K, fp32 partials);
 //   reduce : sums the K splits and stores the result as a hi + lo pair of 16-bit values, so
 //            the intermediate keeps fp32 accuracy through the second MFMA;
@@ -98,7 +98,9 @@ __global__ __launch_bounds__(1024) void sgmv_plan_kernel(const SgmvArgs p)
         const int s = s0 + tid;
         int start = 0, len = 0, adapter = -1;
         if (s < p.n_seg) seg_of(p, s, start, len, adapter);
-        const int nt = (len + TM - 1) / TM;
+        // tiles of a segment: every TM tokens from its start, or (aligned) the pieces between multiples of TM
+        const int lead = p.tile_aligned ? start % TM : 0;
+        const int nt = (lead + len + TM - 1) / TM;
         int v = nt;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
@@ -112,9 +114,11 @@ __global__ __launch_bounds__(1024) void sgmv_plan_kernel(const SgmvArgs p)
         int idx = base + v - nt;
         for (int i = 0; i < nt; i++, idx++) {
             if (idx < p.max_tiles) {
+                const int b = i == 0 ? start : start - lead + i * TM;
+                const int e = start - lead + (i + 1) * TM < start + len ? start - lead + (i + 1) * TM : start + len;
                 p.tile_seg[idx] = s;
-                p.tile_tok0[idx] = start + i * TM;
-                p.tile_ntok[idx] = len - i * TM < TM ? len - i * TM : TM;
+                p.tile_tok0[idx] = b;
+                p.tile_ntok[idx] = e - b;
             }
         }
         __syncthreads();

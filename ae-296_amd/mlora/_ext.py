@@ -53,6 +53,7 @@ SIGNATURES = {
     "mlora_sgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                           _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     "mlora_sgmv_plan": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _i32, _vp, _i64, _vp]),
+    "mlora_sgmv_plan_aligned": (_i32, [_vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i64, _i32, _vp, _i64, _vp]),
     "mlora_sgmv_planned": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                   _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     "mlora_sgmv_multi_workspace_bytes": (_i64, [_i32, _i32, _i32]),

@@ -241,14 +241,18 @@ def _check_segments(seg_start, seg_len, seg_adapter):
 
 
 def plan_prefill(seg_start: torch.Tensor, seg_len: torch.Tensor, seg_adapter: torch.Tensor, T: int,
-                 pool: AdapterPool, workspace: Optional[torch.Tensor] = None, n_proj: int = 1) -> PrefillPlan:
+                 pool: AdapterPool, workspace: Optional[torch.Tensor] = None, n_proj: int = 1,
+                 aligned: bool = False) -> PrefillPlan:
     """Plan a prefill batch once; the plan serves every projection and layer (``sgmv(..., plan=plan)``,
-    ``sgmv_multi(..., plan=plan)`` for up to `n_proj` projections per call)."""
+    ``sgmv_multi(..., plan=plan)``, ``gemm_lora(..., plan)`` for up to `n_proj` projections per call).
+    ``aligned`` cuts the tiles at multiples of 64 tokens (and at segment ends) rather than every 64 tokens of a
+    segment: fewer tiles per 256-row block of ``gemm_lora``, a few more tiles overall."""
     n_seg = _check_segments(seg_start, seg_len, seg_adapter)
     if workspace is None:
         workspace = sgmv_workspace(T, n_seg, seg_start.device, n_proj)
     pool.sync()
-    rc = _ext.lib().mlora_sgmv_plan(
+    plan_fn = _ext.lib().mlora_sgmv_plan_aligned if aligned else _ext.lib().mlora_sgmv_plan
+    rc = plan_fn(
         seg_start.data_ptr(), seg_len.data_ptr(), seg_adapter.data_ptr(), n_seg,
         _ext.ptr(pool.page_tbl), _ext.ptr(pool.rank), _ext.ptr(pool.scaling), T, pool.n_slots, pool.max_pages,
         pool.page_rows, pool.n_pages, pool.max_rank, workspace.data_ptr(), workspace.numel(), _ext.current_stream_ptr())

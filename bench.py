@@ -194,7 +194,7 @@ def bench_f1(args, dev):
     ws = mlora.sgmv_workspace(T, 16, dev, n_proj=len(names))
 
     def fused():
-        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)
+        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws, aligned=True)
         mlora.gemm_lora([y[p] for p in names], [x_in[p] for p in names], [w[p] for p in names], pool, 0, names, plan)
 
     def unfused():

@@ -230,6 +230,16 @@ int mlora_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, const int3
                     const int32_t *page_tbl, const int32_t *rank, const float *scaling,
                     int T, int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
                     void *workspace, int64_t workspace_bytes, void *stream);
+/*
+ * mlora_sgmv_plan with the tiles cut at multiples of 64 tokens (and at segment ends) instead of every 64
+ * tokens from each segment's start.  Valid for every *_planned call; meant for mlora_gemm_lora_planned, whose
+ * 256-row output blocks then meet four tiles (one per 64 rows) except where a segment ends inside a block.
+ * No counterpart in the reference.
+ */
+int mlora_sgmv_plan_aligned(const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
+                            const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                            int T, int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                            void *workspace, int64_t workspace_bytes, void *stream);
 int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b_rows,
                        const int32_t *seg_start, const int32_t *seg_len, const int32_t *seg_adapter, int n_seg,
                        const int32_t *page_tbl, const int32_t *rank, const float *scaling,

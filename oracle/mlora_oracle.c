@@ -297,6 +297,27 @@ int orc_sgmv_plan(const int32_t *seg_start, const int32_t *seg_len, int n_seg, i
     return ORC_OK;
 }
 
+/* The same with the cuts at multiples of `tile` tokens (and at segment ends): segment [start, start + len) gives
+ * the non-empty pieces [max(start, k tile), min(start + len, (k + 1) tile)), k ascending. */
+int orc_sgmv_plan_aligned(const int32_t *seg_start, const int32_t *seg_len, int n_seg, int tile,
+                          int32_t *tile_seg, int32_t *tile_tok0, int32_t *tile_ntok, int32_t *n_tiles)
+{
+    if (tile <= 0) return ORC_EINVAL;
+    int nt = 0;
+    for (int s = 0; s < n_seg; s++) {
+        int b = seg_start[s], end = seg_start[s] + seg_len[s];
+        while (b < end) {
+            int e = (b / tile + 1) * tile;
+            if (e > end) e = end;
+            tile_seg[nt] = s; tile_tok0[nt] = b; tile_ntok[nt] = e - b;
+            nt++;
+            b = e;
+        }
+    }
+    *n_tiles = nt;
+    return ORC_OK;
+}
+
 /* ------------------------------------------------------------------ */
 /* LoRA apply over the paged pool:                                     */
 /*   y[t] = round16( y0[t] + s_a * (x[t] . A_a) . B_a ),  a = adapter   */

@@ -159,15 +159,16 @@ def build_work(chunk_start, chunk_len, chunk_adapter, perm, page_tbl, rank, scal
     return work
 
 
-def sgmv_plan(seg_start, seg_len, tile):
+def sgmv_plan(seg_start, seg_len, tile, aligned=False):
     seg_start = np.ascontiguousarray(seg_start, np.int32)
     seg_len = np.ascontiguousarray(seg_len, np.int32)
-    cap = int(sum((int(l) + tile - 1) // tile for l in seg_len)) + 1
+    cap = int(sum((int(l) + tile - 1) // tile + 1 for l in seg_len)) + 1
     ts = np.zeros(cap, np.int32)
     t0 = np.zeros(cap, np.int32)
     tn = np.zeros(cap, np.int32)
     n = C.c_int32(0)
-    rc = lib().orc_sgmv_plan(_p(seg_start), _p(seg_len), seg_start.size, tile, _p(ts), _p(t0), _p(tn), C.byref(n))
+    fn = lib().orc_sgmv_plan_aligned if aligned else lib().orc_sgmv_plan
+    rc = fn(_p(seg_start), _p(seg_len), seg_start.size, tile, _p(ts), _p(t0), _p(tn), C.byref(n))
     _check(rc, "sgmv_plan")
     return ts[:n.value].copy(), t0[:n.value].copy(), tn[:n.value].copy()
 

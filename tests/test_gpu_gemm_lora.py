@@ -37,13 +37,13 @@ def _tok_of(start, lens, adapters, T):
     return tok
 
 
-def _run(pp, x_bits, w_bits, seg, T):
+def _run(pp, x_bits, w_bits, seg, T, aligned=False):
     pool = upload_pool(pp)
     x = bits_to_torch(x_bits, pp.dtype, "cuda")
     w = bits_to_torch(w_bits, pp.dtype, "cuda")
     y = torch.full((T, pp.hout), float("nan"), dtype=tdtype(pp.dtype), device="cuda")
     ss, sl, sa = (torch.from_numpy(a).cuda() for a in seg)
-    plan = plan_prefill(ss, sl, sa, T, pool)
+    plan = plan_prefill(ss, sl, sa, T, pool, aligned=aligned)
     gemm_lora([y], [x], [w], pool, 0, ["p"], plan)
     torch.cuda.synchronize()
     return torch_to_bits(y)
@@ -75,6 +75,8 @@ def test_gemm_lora_vs_oracle(name, lens, gaps, tail, ranks, hin, hout, dtype):
     say(f"gemm_lora {name}")
     got = _run(pp, x, w, (ss, sl, sa), T)
     assert_close_bits(got, _oracle(pp, x, w, tok), dtype, name)
+    say(f"gemm_lora {name}, tiles cut at multiples of 64")
+    assert_close_bits(_run(pp, x, w, (ss, sl, sa), T, aligned=True), _oracle(pp, x, w, tok), dtype, name + " aligned")
     # much closer than the tolerance: within one 16-bit ulp of the fp64 result (+ fp32 accumulation noise)
     want64 = f32_of(_oracle(pp, x, w, tok, acc64=True), dtype).astype(np.float64)
     err = np.abs(f32_of(got, dtype) - want64)
@@ -97,6 +99,7 @@ def test_gemm_lora_integer_inputs_bit_exact():
     assert np.abs(f32_of(want, FP16)).max() < 2048
     say("gemm_lora integer-valued inputs")
     assert np.array_equal(_run(pp, x, w, (ss, sl, sa), T), want)
+    assert np.array_equal(_run(pp, x, w, (ss, sl, sa), T, aligned=True), want)
 
 
 @pytest.mark.parametrize("dtype", [FP16, BF16])
@@ -189,3 +192,28 @@ def test_gemm_lora_config4_width_against_library_products():
     assert float(delta.float().abs().max()) > 0.05                      # the delta is not negligible here
     # three bf16 roundings (y, base, delta) apart at most
     assert bool(((y.float() - yb.float() - delta.float()).abs() <= 2.0 ** -7 * (ref.abs() + delta.float().abs()) + 1e-4).all())
+
+
+@pytest.mark.parametrize("aligned", [False, True])
+def test_plan_tile_list_matches_oracle(aligned):
+    """The tile list the plan kernel writes (first words of the workspace: segment, first token and token count
+    per tile, then the count) is the oracle's, bit for bit, in both cutting modes; and SGMV gives the same
+    result with either plan."""
+    rng = np.random.default_rng(91)
+    lens = rng.integers(0, 300, 37).astype(np.int32)
+    gaps = (rng.integers(0, 2, 37) * rng.integers(0, 50, 37)).astype(np.int32)
+    ss, sl, sa, T = _layout(lens, gaps, rng.integers(-1, 3, 37))
+    T += 5
+    pp = PagedPool(rng, [16, 8, 4], 64, 64, page_rows=8, dtype=FP16)
+    pool = upload_pool(pp)
+    say(f"plan tile list aligned={aligned}")
+    plan = plan_prefill(*(torch.from_numpy(a).cuda() for a in (ss, sl, sa)), T, pool, aligned=aligned)
+    torch.cuda.synchronize()
+    want_s, want_t0, want_n = orc.sgmv_plan(ss, sl, 64, aligned=aligned)
+    max_tiles = T // 64 + 2 * len(lens) + 1
+    words = plan.workspace[:(3 * max_tiles + 1) * 4].cpu().numpy().view(np.int32)
+    n = int(words[3 * max_tiles])
+    assert n == len(want_s)
+    assert np.array_equal(words[:n], want_s)
+    assert np.array_equal(words[max_tiles:max_tiles + n], want_t0)
+    assert np.array_equal(words[2 * max_tiles:2 * max_tiles + n], want_n)

@@ -144,6 +144,26 @@ def test_sgmv_plan_brute_force():
     assert np.all(covered == 1)
 
 
+def test_sgmv_plan_aligned_brute_force():
+    """Aligned cuts: every token of every segment in exactly one tile, no tile crosses a multiple of 64 or a
+    segment end, tiles in token order within a segment, and as few tiles as that allows."""
+    rng = np.random.default_rng(6)
+    lens = rng.integers(0, 400, 29)
+    gaps = rng.integers(0, 3, 29) * rng.integers(0, 70, 29)
+    starts = np.cumsum(gaps) + np.concatenate([[0], np.cumsum(lens)[:-1]])
+    ts, t0, tn = orc.sgmv_plan(starts, lens, 64, aligned=True)
+    want = []
+    for s in range(29):
+        toks = np.arange(int(starts[s]), int(starts[s] + lens[s]))
+        for k in np.unique(toks // 64):                       # ascending
+            part = toks[toks // 64 == k]
+            want.append((s, int(part[0]), len(part)))
+    assert list(zip(ts.tolist(), t0.tolist(), tn.tolist())) == want
+    assert all(a // 64 == (a + n - 1) // 64 and 1 <= n <= 64 for _, a, n in want)
+    # never more than one tile more per segment end than the unaligned cut
+    assert len(want) <= len(orc.sgmv_plan(starts, lens, 64)[0]) + int((lens > 0).sum())
+
+
 @pytest.mark.parametrize("batch,tkn,cap", [(1, 64, 8), (3, 20, 8), (2, 8, 8), (4, 1, 16), (2, 17, 16), (1, 256, 8)])
 def test_cpu_chunk_plan_matches_reference_formulas(batch, tkn, cap):
     req, tok0, ntok = orc.cpu_chunk_plan(batch, tkn, cap)
