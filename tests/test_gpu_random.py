@@ -88,3 +88,46 @@ def test_random_prefill(seed):
     assert torch.equal(y2, y3)
     covered = tok >= 0
     assert np.array_equal(torch_to_bits(y2)[~covered], y0[~covered])
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_gemm_lora(seed):
+    """Base projection + LoRA in one pass on random shapes: few and many K steps with and without a partial one,
+    ragged row and column tiles, empty and tiny segments, gaps, adapter-less segments, both tile cuts."""
+    from mlora import gemm_lora
+    from oracle import oracle as orc
+    rng = np.random.default_rng(3000 + seed)
+    dtype = BF16 if seed % 2 else FP16
+    N = int(rng.integers(1, 9))
+    ranks = rng.choice([1, 4, 8, 16, 24, 32, 48, 64], N)
+    if seed % 3 == 0:
+        ranks = np.minimum(ranks, 16)
+    elif seed % 3 == 1:
+        ranks = np.minimum(ranks, 32)
+    hin = int(rng.choice([8, 40, 64, 96, 136, 256, 328, 520]))
+    hout = int(rng.choice([8, 72, 256, 264, 520]))
+    n_seg = int(rng.integers(1, 9))
+    lens = rng.choice([0, 1, 5, 63, 64, 65, 130, 257], n_seg)
+    gaps = rng.choice([0, 0, 3], n_seg)
+    starts = np.cumsum(np.r_[gaps[0], lens[:-1] + gaps[1:]]).astype(np.int32)
+    T = int(starts[-1] + lens[-1] + rng.choice([0, 2]))
+    if T == 0:
+        T, lens[0] = 4, 4
+    adapters = rng.integers(-1, N, n_seg).astype(np.int32)
+    tok = np.full(T, -1, np.int32)
+    for s, l, a in zip(starts, lens, adapters):
+        tok[s:s + l] = a
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=dtype)
+    pool = upload_pool(pp)
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype)
+    w = bits_of((rng.standard_normal((hin, hout)) / np.sqrt(hin)).astype(np.float32), dtype)
+    want = orc.gemm_lora_paged(x, w, pp.a_rows, pp.b_rows, tok, pp.page_tbl, pp.page_tbl, pp.ranks, pp.scaling,
+                               pp.page_rows, dtype)
+    d = [torch.from_numpy(np.asarray(a, np.int32)).cuda() for a in (starts, lens, adapters)]
+    xt, wt = bits_to_torch(x, dtype, "cuda"), bits_to_torch(w, dtype, "cuda")
+    for aligned in (False, True):
+        say(f"random gemm_lora seed={seed} T={T} segs={n_seg} {hin}x{hout} max_rank={pool.max_rank} aligned={aligned}")
+        y = torch.full((T, hout), float("nan"), dtype=xt.dtype, device="cuda")
+        gemm_lora([y], [xt], [wt], pool, 0, ["p"], plan_prefill(d[0], d[1], d[2], T, pool, aligned=aligned))
+        torch.cuda.synchronize()
+        assert_close_bits(torch_to_bits(y), want, dtype, f"seed {seed} aligned {aligned}")
