@@ -505,9 +505,12 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
+                for (int e = 0; e < 16; e += 2) {
+                    // two rows of one column, converted as a pair by the hardware (round to nearest even)
+                    const uint32_t u = pack2<DT>(acc[i][j][e], acc[i][j][e + 1]);
                     const int row = 8 * (e >> 2) + 4 * lh + (e & 3);
-                    *(lds_vu16 *)(so + row * OPITCH + (j * 32 + l32) * 2) = (uint16_t)cvt16<DT>(acc[i][j][e]);
+                    *(lds_vu16 *)(so + row * OPITCH + (j * 32 + l32) * 2) = (uint16_t)u;
+                    *(lds_vu16 *)(so + (row + 1) * OPITCH + (j * 32 + l32) * 2) = (uint16_t)(u >> 16);
                 }
 #pragma unroll
             for (int q = 0; q < 8; q++) {
