@@ -61,3 +61,45 @@ def test_graph_replays_match_eager():
         assert scratch.isfinite()
         for got, w in zip(y_dec + y_pre, want):
             assert torch.equal(got, w), rep
+
+
+def test_graph_replays_of_the_one_pass_projection_match_eager():
+    """The base projection + LoRA call (plan, shrink, scaled reduce, GEMM) under a HIP graph: every replay gives the
+    eager result bit for bit, with eager work in between."""
+    from mlora import gemm_lora
+    rng = np.random.default_rng(92)
+    ranks = [16, 64, 32]
+    hin, hout = 320, 520
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=FP16)
+    pool = upload_pool(pp)
+    lens = np.array([130, 7, 200, 64], np.int32)
+    starts = np.array([2, 132, 140, 345], np.int32)
+    T = 420
+    ss, sl = torch.from_numpy(starts).cuda(), torch.from_numpy(lens).cuda()
+    sa = torch.from_numpy(np.array([1, -1, 0, 2], np.int32)).cuda()
+    x = torch.randn(T, hin, device="cuda").half()
+    w = (torch.randn(hin, hout, device="cuda") / hin ** 0.5).half()
+    y = torch.zeros(T, hout, device="cuda").half()
+    pplan = plan_prefill(ss, sl, sa, T, pool, aligned=True)
+
+    def step():
+        plan_prefill(ss, sl, sa, T, pool, workspace=pplan.workspace, aligned=True)
+        gemm_lora([y], [x], [w], pool, 0, ["p"], pplan)
+
+    say("graph: eager one-pass projection")
+    step()
+    torch.cuda.synchronize()
+    want = y.clone()
+    assert bool(torch.isfinite(want.float()).all()) and not torch.equal(want, torch.mm(x, w))   # the delta is in there
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for rep in range(4):
+        y.fill_(float(rep))
+        scratch = (torch.randn(1 << 20, device="cuda") * 2).sum()
+        torch.cuda.synchronize()
+        say(f"graph: one-pass projection replay {rep}")
+        g.replay()
+        torch.cuda.synchronize()
+        assert scratch.isfinite()
+        assert torch.equal(y, want), rep
