@@ -100,9 +100,10 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     __shared__ __attribute__((aligned(16))) unsigned char smem1[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char smem2[STAGE];
     __shared__ __attribute__((aligned(16))) unsigned char smem3[STAGE];
-    __shared__ unsigned long long s_mask[G_NT / 64];
-    __shared__ int s_list[G_NT + 1];               // plan tiles (of the 256 looked at) that overlap this row block; [G_NT] = how many
-    __shared__ int s_rows[4][MAX_RANK];            // row of every rank row of the (up to four) plan tiles being applied
+    __shared__ unsigned long long s_mask[2 * (G_NT / 64)];
+    __shared__ int s_list[G_NT + 1];               // first plan tile of every run (of the 256 tiles looked at); [G_NT] = how many runs
+    __shared__ int s_last[G_NT];                   // last plan tile of every run
+    __shared__ int s_rows[4][MAX_RANK];            // row of every rank row of the (up to four) runs being applied
     __shared__ int s_span[4][2];                   // their first and one-past-last row, relative to this row block
 
     // ---- which projection, which tile.  Workgroups go to the 8 XCDs round-robin by id; every XCD works
@@ -128,39 +129,59 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     const int l32 = lane & 31, lh = lane >> 5;
     const int T = p.T, hin = pj.hin, hout = pj.hout;
 
-    // Which plan tiles (at most 64 consecutive tokens of one adapter) overlap this row block: asked now, for the
-    // first 256 tiles of the plan, so that the answer is there when the K loop ends (one bit per tile).
-    auto tile_hits = [&](int ti, int n_plan) {
-        if (ti >= n_plan) return false;
+    // Which rows of this block get which adapter.  A plan tile is at most 64 consecutive tokens of one segment;
+    // consecutive tiles of one segment that overlap the block form a "run" (one adapter, one contiguous row
+    // range), which is what the expand works on.  Asked now, for the first 256 tiles of the plan, so that the
+    // answer is there when the K loop ends.  tile_hits: does tile ti overlap the block (and have an adapter);
+    // its segment goes to `seg`.
+    auto tile_hits = [&](int ti, int n_plan, int &seg) {
+        seg = -1;
+        if (ti < 0 || ti >= n_plan) return false;
         const int32_t *rec = p.tile_rec + (size_t)ti * TILE_WORDS;
         const int4 h = *reinterpret_cast<const int4 *>(rec);             // tokens, adapter, rank, scaling
         const int tok0 = rec[4];
+        seg = rec[5];
         return h.y >= 0 && h.z > 0 && h.x > 0 && tok0 >= 0 && tok0 + h.x <= T && tok0 < m0 + GM && tok0 + h.x > m0;
     };
     const int n_plan = p.lora ? p.n_tiles[0] : 0;
-    // s_list = the tiles among plan tiles b0 .. b0 + 255 that overlap this row block, in order (two barriers inside)
+    // s_list / s_last = first and last tile of every run among plan tiles b0 .. b0 + 255, in order (a run that
+    // crosses the window's end is cut there); s_list[G_NT] = how many (two barriers inside)
     auto list_tiles = [&](int b0) {
-        const bool hit = tile_hits(b0 + tid, n_plan);
-        const unsigned long long bal = __ballot(hit);
-        if (lane == 0) s_mask[wave] = bal;
+        const int ti = b0 + tid;
+        int seg, segp, segn;
+        const bool hit = tile_hits(ti, n_plan, seg);
+        const bool hitp = tid > 0 && tile_hits(ti - 1, n_plan, segp);
+        const bool hitn = tid < G_NT - 1 && tile_hits(ti + 1, n_plan, segn);
+        const bool head = hit && !(hitp && segp == seg), tail = hit && !(hitn && segn == seg);
+        const unsigned long long balh = __ballot(head), balt = __ballot(tail);
+        if (lane == 0) { s_mask[wave] = balh; s_mask[G_NT / 64 + wave] = balt; }
         __syncthreads();
-        int before = 0;
-        for (int w4 = 0; w4 < wave; w4++) before += __builtin_popcountll(s_mask[w4]);
-        if (hit) s_list[before + __builtin_popcountll(bal & ((1ull << lane) - 1))] = b0 + tid;
-        if (tid == G_NT - 1) s_list[G_NT] = before + __builtin_popcountll(bal);
+        int beforeh = 0, beforet = 0;
+        for (int w4 = 0; w4 < wave; w4++) {
+            beforeh += __builtin_popcountll(s_mask[w4]);
+            beforet += __builtin_popcountll(s_mask[G_NT / 64 + w4]);
+        }
+        const unsigned long long below = (1ull << lane) - 1;
+        if (head) s_list[beforeh + __builtin_popcountll(balh & below)] = ti;
+        if (tail) s_last[beforet + __builtin_popcountll(balt & below)] = ti;
+        if (tid == G_NT - 1) s_list[G_NT] = beforeh + __builtin_popcountll(balh);
         __syncthreads();
     };
-    // thread (q, j) = (tid / 64, tid % 64) copies rank row j's row index of tile s_list[base + q] into LDS
+    // thread (q, j) = (tid / 64, tid % 64) copies rank row j's row index of run base + q into LDS, and its row span
     auto fill_rows = [&](int base, int count) {
         const int q = tid >> 6, j = tid & 63;
         if (base + q < count) {
             const int32_t *rec = p.tile_rec + (size_t)s_list[base + q] * TILE_WORDS;
             s_rows[q][j] = rec[TILE_ROWS_AT + j];
-            if (j < 2) s_span[q][j] = rec[4] - m0 + (j ? rec[0] : 0);
+            if (j == 0) s_span[q][0] = rec[4] - m0;
+            if (j == 1) {
+                const int32_t *recl = p.tile_rec + (size_t)s_last[base + q] * TILE_WORDS;
+                s_span[q][1] = recl[4] + recl[0] - m0;
+            }
         }
     };
     if (p.lora) {
-        // the first four overlapping tiles: their records are fetched now, behind the K loop
+        // the first four runs: their records are fetched now, behind the K loop
         list_tiles(0);
         fill_rows(0, s_list[G_NT]);                // visible after the barrier that opens the K loop
     }
