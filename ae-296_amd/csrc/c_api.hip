@@ -358,7 +358,7 @@ namespace {
 
 constexpr int SG_TM = 64;   // tokens per tile, as in sgmv_prefill.hip
 
-struct SgmvWs { int max_tiles; int ksplit; size_t off_rec, off_proj, per_proj, off_hi, off_lo, total; };
+struct SgmvWs { int max_tiles; int ksplit; int ks_cap; size_t off_rec, off_proj, per_proj, off_hi, off_lo, total; };
 
 // Workspace: the plan (tile list, tile records: depends on T and n_seg only), then per projection the
 // K-split partial sums and the hi / lo halves of their sum.
@@ -372,13 +372,16 @@ SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
     const long long target = n_proj > 1 ? 2048 : 768;
     long long ks = (target + per_split - 1) / per_split;
     w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : (int)ks);
+    // a projection with a longer K than the others of its call gets proportionally more splits (up to three
+    // times as many, at most 8), so that every shrink workgroup walks about the same number of columns
+    w.ks_cap = n_proj > 1 ? (3 * w.ksplit < 8 ? 3 * w.ksplit : 8) : w.ksplit;
     size_t off = ((size_t)w.max_tiles * 3 + 4) * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
     w.off_rec = off;
     off += (size_t)w.max_tiles * 80 * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
     w.off_proj = off;
-    w.off_hi = (size_t)w.ksplit * T * MLORA_MAX_RANK * sizeof(float);
+    w.off_hi = (size_t)w.ks_cap * T * MLORA_MAX_RANK * sizeof(float);
     w.off_lo = w.off_hi + (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t);
     w.per_proj = (w.off_lo + (size_t)T * MLORA_MAX_RANK * sizeof(uint16_t) + 255) & ~(size_t)255;
     w.total = off + w.per_proj * n_proj;
@@ -393,12 +396,15 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
     a.n_tiles = ip + 3 * (size_t)w.max_tiles;
     a.tile_rec = reinterpret_cast<int32_t *>(base + w.off_rec);
     a.max_tiles = w.max_tiles;
+    int hin_min = a.pr[0].hin;
+    for (int p = 1; p < a.n_proj; p++) hin_min = a.pr[p].hin < hin_min ? a.pr[p].hin : hin_min;
     for (int p = 0; p < a.n_proj; p++) {
         char *pb = base + w.off_proj + w.per_proj * p;
         a.pr[p].v = reinterpret_cast<float *>(pb);
         a.pr[p].vhi = reinterpret_cast<uint16_t *>(pb + w.off_hi);
         a.pr[p].vlo = reinterpret_cast<uint16_t *>(pb + w.off_lo);
-        a.pr[p].ksplit = w.ksplit;
+        int ks = (int)(((long long)w.ksplit * a.pr[p].hin + hin_min / 2) / (hin_min > 0 ? hin_min : 1));
+        a.pr[p].ksplit = ks < w.ksplit ? w.ksplit : (ks > w.ks_cap ? w.ks_cap : ks);
         // 512 columns per expand workgroup amortise the V operand; fewer when that leaves the chip idle
         int cols = 512;
         if (a.n_proj == 1)
