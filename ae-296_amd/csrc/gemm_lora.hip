@@ -47,11 +47,6 @@ __device__ __forceinline__ float16_t mfma32(const uint4 &a, const uint4 &b, floa
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
 }
 
-// The B operand of a 32x32x16 MFMA out of a row-major [k][n] LDS tile: lane (n = lane % 32, k group = lane / 32)
-// needs rows k0 + 8 * (lane / 32) + 0..7 of column n0 + lane % 32.  Each transposing read (ds_read_b64_tr_b16)
-// serves a 16-lane group: lane i of the group addresses row i / 4, columns 4 * (i % 4) .. + 3, and receives the
-// four rows of column i.
-
 // ------------------------------------------------------------------ scaled reduce
 // vhi + vlo [t][0..RMAX) = s_a * sum over the K splits of the shrink partials, for the tokens of one plan
 // tile (the scaling is folded in here because the GEMM accumulators also hold the base product).
@@ -272,7 +267,10 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
             b_at[j] = (unsigned)(krow * (GN * 2) + c * 16 + (m & 1) * 8);
         }
     }
-    // W operands of one K = 16 slice out of a [k rows][512 bytes] swizzled tile at `tile`
+    // W operands of one K = 16 slice out of a [k rows][512 bytes] swizzled tile at `tile`.  The W-side operand of
+    // a 32x32x16 MFMA: lane (n = lane % 32, k group = lane / 32) needs rows 8 * (lane / 32) + 0..7 of column n.
+    // Each transposing read (ds_read_b64_tr_b16) serves a 16-lane group: lane i of the group addresses row
+    // i / 4, columns 4 * (i % 4) .. + 3, and receives the four rows of column i; two reads give the eight rows.
     auto w_frags = [&](const unsigned char *tile, int kk, uint4 (&bf)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -400,8 +398,8 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     }
     if (ns * GK < hin) {
         // Partial last K step: through registers, with chunks of x and rows of W beyond hin replaced by zeros,
-        // parked in the same swizzled layout.  Every wavefront has passed the last barrier of the pipeline and
-        // stage 1 is not being read (the last step read stage (ns - 1) % 4; use the one after it).
+        // parked in the same swizzled layout, in the stage after the one the last full step read (some wavefronts
+        // may still be reading that one; the one after it was released four steps ago).
         unsigned char *st = (ns & 3) == 0 ? smem : (ns & 3) == 1 ? smem1 : (ns & 3) == 2 ? smem2 : smem3;
         const int ncc = hin >> 3;
 #pragma unroll
