@@ -16,6 +16,7 @@
 // records in use come first in launch order and the empty tail costs no waiting.
 //
 // Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
+#include <type_traits>
 #include "mlora_args.hpp"
 #include "mlora_dev.hpp"
 
@@ -33,12 +34,26 @@ __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
     return r;
 }
 
+// Slices of the launch's width (Slices<RMAX>::KSC) that one shrink workgroup takes, by the rank bucket of
+// its item (more than 32, 17..32, 9..16, at most 8 rank rows): the bytes of a workgroup grow with
+// rank x width, so an item of low rank in a launch sized for rank 64 takes wider slices.
+template <int RMAX> struct SliceFactor;
+template <> struct SliceFactor<16> { static constexpr int F16 = 1, F8 = 1, F4 = 1, F2 = 1; };
+template <> struct SliceFactor<32> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
+template <> struct SliceFactor<64> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
+template <int RMAX>
+__device__ __forceinline__ int slice_factor(int r)
+{
+    using SF = SliceFactor<RMAX>;
+    return r > 32 ? SF::F16 : (r > 16 ? SF::F8 : (r > 8 ? SF::F4 : SF::F2));
+}
+
 // Shrink of one (item, projection, column slice) over the first 4 * NR rank rows (NR per 16-lane
 // row).  The caller picks the smallest NR that covers the item's rank, so an adapter of rank 8 in a
 // pool that goes up to rank 64 issues loads for 8 rows, not 64.
 template <int DT, int G, int RMAX, int KSC, int NR>
 __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__restrict__ rows, const int (&tok)[G],
-                                            int r, int proj, int ks, float (&s_part)[4][G][RMAX])
+                                            int r, int proj, int ks, int slot, float (&s_part)[4][G][RMAX])
 {
     constexpr int NW = 4;
     constexpr int STEPS = KSC / 64;                             // 16-chunk steps per wavefront
@@ -119,7 +134,7 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
             float s = 0.f;
 #pragma unroll
             for (int wv = 0; wv < NW; wv++) s += s_part[wv][k][j];
-            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + ks) * RMAX + j] = s;
+            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + slot) * RMAX + j] = s;
         }
     }
 }
@@ -148,15 +163,23 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     }
     const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
 
-    // r is uniform over the workgroup: a scalar branch, no divergence.
+    // r is uniform over the workgroup: a scalar branch, no divergence.  An item of a lower rank bucket
+    // takes F consecutive slices in one workgroup (the others of the F leave at once) and stores its sums
+    // in the slot of the first.
+    auto go = [&](auto nr_tag, auto f_tag) {
+        constexpr int NR = decltype(nr_tag)::value, F = decltype(f_tag)::value;
+        if (ks % F) return;
+        shrink_rows<DT, G, RMAX, KSC * F, NR>(p, rows, tok, r, proj, ks / F, ks, s_part);
+    };
+    using SF = SliceFactor<RMAX>;
     if constexpr (RMAX >= 64) {
-        if (r > 32) { shrink_rows<DT, G, RMAX, KSC, 16>(p, rows, tok, r, proj, ks, s_part); return; }
+        if (r > 32) { go(std::integral_constant<int, 16>{}, std::integral_constant<int, SF::F16>{}); return; }
     }
     if constexpr (RMAX >= 32) {
-        if (r > 16) { shrink_rows<DT, G, RMAX, KSC, 8>(p, rows, tok, r, proj, ks, s_part); return; }
+        if (r > 16) { go(std::integral_constant<int, 8>{}, std::integral_constant<int, SF::F8>{}); return; }
     }
-    if (r > 8) { shrink_rows<DT, G, RMAX, KSC, 4>(p, rows, tok, r, proj, ks, s_part); return; }
-    shrink_rows<DT, G, RMAX, KSC, 2>(p, rows, tok, r, proj, ks, s_part);
+    if (r > 8) { go(std::integral_constant<int, 4>{}, std::integral_constant<int, SF::F4>{}); return; }
+    go(std::integral_constant<int, 2>{}, std::integral_constant<int, SF::F2>{});
 }
 
 template <int DT, int G, int RMAX, int KSC, int NTE>
@@ -235,12 +258,13 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 
     // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
     const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
+    const int kstep = slice_factor<RMAX>(r);                   // the shrink filled every kstep-th slot
     for (int e = tid; e < G * RMAX; e += NT) {
         const int k = e / RMAX, j = e - k * RMAX;
         float s = 0.f;
         if (j < r && tok[k] >= 0) {
             const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
-            for (int ks = 0; ks < n_ks; ks++) s += src[(size_t)ks * RMAX];
+            for (int ks = 0; ks < n_ks; ks += kstep) s += src[(size_t)ks * RMAX];
         }
         s_v[k][j] = s * scale;
     }
