@@ -95,6 +95,42 @@ def cpu_baseline(seconds=12.0):
     return out
 
 
+def cpu_baseline_prefill(with_base, seconds=10.0):
+    """The oracle (scalar C, one core) on a bounded sample of the config-4 prefill: one segment (128 tokens, or
+    32 with the base product) on one rank-64 adapter, q projection 5120 -> 5120, bf16 -- the LoRA delta added
+    into y (`with_base` False, the SGMV step) or y = x W + delta (`with_base` True).  Reported in the GPU
+    line's unit (TFLOP/s)."""
+    import numpy as np
+    from oracle import oracle as orc
+    rng = np.random.default_rng(1004)
+    Ts, H, r, page_rows = (32 if with_base else 128), 5120, 64, 8
+    n_pages = r // page_rows
+    bf = lambda a: orc.to_bits(a.astype(np.float32), orc.BF16)
+    x = bf(rng.standard_normal((Ts, H)))
+    a_rows = bf(rng.standard_normal((r, H)) * 0.02)
+    b_rows = bf(rng.standard_normal((r, H)) * 0.02)
+    tbl = np.arange(n_pages, dtype=np.int32)[None, :]
+    tok = np.zeros(Ts, np.int32)
+    rank, scaling = np.array([r], np.int32), np.array([0.5], np.float32)
+    if with_base:
+        w = bf(rng.standard_normal((H, H)) / H ** 0.5)
+        fn = lambda: orc.gemm_lora_paged(x, w, a_rows, b_rows, tok, tbl, tbl, rank, scaling, page_rows, orc.BF16)
+        flops = 2.0 * Ts * H * H + 2.0 * r * 2 * H * Ts
+    else:
+        y0 = bf(rng.standard_normal((Ts, H)))
+        fn = lambda: orc.lora_apply_paged(x, a_rows, b_rows, tok, tbl, tbl, rank, scaling, page_rows, orc.BF16, y0=y0)
+        flops = 2.0 * r * 2 * H * Ts
+    fn()
+    n, t0 = 0, time.perf_counter()
+    while n == 0 or time.perf_counter() - t0 < seconds:
+        fn()
+        n += 1
+    dt = time.perf_counter() - t0
+    return {"value": flops * n / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": f"one {Ts}-token segment, one rank-64 adapter, q projection 5120->5120, bf16"
+                      f"{', with the base product' if with_base else ''}: {n} repetitions in {dt:.1f} s on one core"}
+
+
 def bench_c4(args, dev):
     """Prefill SGMV, config 4: Llama-13B shapes (hidden 5120, MLP 13824), 16 requests with prompt lengths
     U[128, 1024], each bound to one of 32 rank-64 adapters, bf16, tokens packed per request.  One step =
@@ -159,7 +195,7 @@ def bench_c4(args, dev):
                         "traffic": None if args.fused else MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
                                   "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
                         "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
-           "cpu_baseline": None}
+           "cpu_baseline": None if args.no_cpu else cpu_baseline_prefill(False)}
     print(json.dumps(out), flush=True)
 
 
@@ -237,7 +273,7 @@ def bench_f1(args, dev):
                         "frac": tflops / MFMA_PEAK_BF16_TFLOPS, "traffic": None,
                         "kernel": "sgmv shrink + scaled reduce + gemm_lora_kernel (one launch over the 7 projections)",
                         "flops_per_step": flops},
-           "cpu_baseline": None}
+           "cpu_baseline": None if args.no_cpu else cpu_baseline_prefill(True)}
     print(json.dumps(out), flush=True)
 
 
