@@ -216,7 +216,8 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         }
     }
     // ---- decode work records, in launch order: workgroup b of a projection reads record b.
-    // Consecutive chunks go to the same XCD (workgroups are dealt to the 8 XCDs round-robin).
+    // Consecutive chunks go to the same XCD (workgroups are dealt to the 8 XCDs round-robin).  Batches
+    // beyond 2048 tokens (chunk headers not in LDS) keep plain chunk order.
     if (g.work) {
         __shared__ int s_nchunks;
         if (tid == GATHER_NT - 1) s_nchunks = ch_incl;
@@ -224,6 +225,30 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         const int n_chunks = s_nchunks;
         const int per_xcd = (n_chunks + 7) >> 3;
         if constexpr (LDS_HDR) {
+            // Within the range of chunks that goes to one XCD the records are written in order of falling rank
+            // (ties keep chunk order, so the chunks of one adapter stay next to each other): the workgroups of
+            // the wide items are then dispatched first and the narrow ones fill in behind them.  A counting sort:
+            // chunks per (XCD, rank), then one thread per (XCD, rank) places its chunks.
+            __shared__ int s_ord[MAXT];
+            __shared__ int s_cntx[8][MAX_RANK + 1];
+            int differs = 0;                     // a pool of one rank keeps chunk order and skips the sort
+            for (int c = tid; c < n_chunks; c += GATHER_NT) differs |= (s_chdr[c] >> (TOK_BITS + 4)) != (s_chdr[0] >> (TOK_BITS + 4));
+            for (int i = tid; i < 8 * (MAX_RANK + 1); i += GATHER_NT) (&s_cntx[0][0])[i] = 0;
+            const bool mixed = __syncthreads_or(differs) != 0;
+            if (mixed)
+                for (int c = tid; c < n_chunks; c += GATHER_NT) atomicAdd(&s_cntx[c / per_xcd][s_chdr[c] >> (TOK_BITS + 4)], 1);
+            __syncthreads();
+            if (mixed && tid < 8 * (MAX_RANK + 1)) {
+                const int xcd = tid / (MAX_RANK + 1), rk = tid - xcd * (MAX_RANK + 1);
+                if (s_cntx[xcd][rk] > 0) {
+                    int at = xcd * per_xcd;
+                    for (int r2 = rk + 1; r2 <= MAX_RANK; r2++) at += s_cntx[xcd][r2];
+                    const int lo = xcd * per_xcd, hi = lo + per_xcd < n_chunks ? lo + per_xcd : n_chunks;
+                    for (int c = lo; c < hi; c++)
+                        if ((s_chdr[c] >> (TOK_BITS + 4)) == rk) s_ord[at++] = c;
+                }
+            }
+            __syncthreads();
             // 16 bytes per step: header quad, two token quads, a zero quad, then 16 quads of row indices.
             constexpr int QPR = WORK_WORDS / 4;
             int4 *out = reinterpret_cast<int4 *>(g.work);
@@ -232,9 +257,10 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
 #pragma unroll 4
             for (int q = tid; q < quads; q += GATHER_NT) {
                 const int b = q / QPR, w4 = q - b * QPR;
-                const int c = (b & 7) * per_xcd + (b >> 3);
+                const int pos = (b & 7) * per_xcd + (b >> 3);
                 int4 v = make_int4(0, w4 == 0 ? -1 : 0, 0, 0);
-                if ((b >> 3) < per_xcd && c < n_chunks) {
+                if ((b >> 3) < per_xcd && pos < n_chunks) {
+                    const int c = mixed ? s_ord[pos] : pos;
                     const int hdr = s_chdr[c];
                     const int start = hdr & (int)tmask, len = (hdr >> TOK_BITS) & 15, rk = hdr >> (TOK_BITS + 4);
                     int a = (int)(s_key[start] >> TOK_BITS);

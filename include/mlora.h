@@ -90,8 +90,11 @@ int mlora_version(void);
  *                       adapter-less tokens in pieces of <= group with adapter -1
  *   counters [MLORA_CNT_WORDS]
  *   work [MLORA_WORK_CAP(T) * MLORA_WORK_WORDS]  (optional, may be NULL) the chunks as decode work
- *                       records in launch order: chunk c is record (c mod P) * 8 + c / P with
- *                       P = ceil(n_chunks / 8), so consecutive chunks run on one XCD.  Record words:
+ *                       records in launch order: position c of the chunk list is record
+ *                       (c mod P) * 8 + c / P with P = ceil(n_chunks / 8), so a range of P consecutive
+ *                       chunks runs on one XCD.  For T <= 2048 the chunks of each such range are placed by
+ *                       falling rank (ties in chunk order), which starts the workgroups of wide items
+ *                       first; the chunk_* arrays keep chunk order.  Record words:
  *                       [0] tokens (0 = empty record) [1] adapter [2] rank [3] scaling (float bits)
  *                       [4..11] token ids [12..15] 0 [16..79] row of rank row j in a rows slab, -1 if
  *                       j >= rank or the page id is outside [0, n_pages).

@@ -255,12 +255,33 @@ int orc_build_work(const int32_t *chunk_start, const int32_t *chunk_len, const i
         for (int i = 0; i < ORC_WORK_WORDS; i++) w[i] = 0;
         w[1] = -1;
     }
+    /* Batches of at most 2048 tokens (work_cap <= 2048): inside the range of chunks that goes to one XCD the
+     * records follow falling rank, ties in chunk order (a stable insertion sort per range). */
+    int *ord = (int *)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(int));
+    int *crk = (int *)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(int));
+    if (!ord || !crk) { free(ord); free(crk); return ORC_EINVAL; }
     for (int c = 0; c < n_chunks; c++) {
-        int b = (c % per_xcd) * 8 + c / per_xcd;
+        int a = chunk_adapter[c], rk = 0;
+        if (a >= 0) { rk = rank[a]; if (rk < 0) rk = 0; if (rk > 64) rk = 64; }
+        crk[c] = rk;
+        ord[c] = c;
+    }
+    if (work_cap <= 2048) {
+        for (int lo = 0; lo < n_chunks; lo += per_xcd) {
+            int hi = lo + per_xcd < n_chunks ? lo + per_xcd : n_chunks;
+            for (int i = lo + 1; i < hi; i++) {
+                int c = ord[i], j = i;
+                while (j > lo && crk[ord[j - 1]] < crk[c]) { ord[j] = ord[j - 1]; j--; }
+                ord[j] = c;
+            }
+        }
+    }
+    for (int pos = 0; pos < n_chunks; pos++) {
+        int c = ord[pos];
+        int b = (pos % per_xcd) * 8 + pos / per_xcd;
         int32_t *w = work + (size_t)b * ORC_WORK_WORDS;
         int a = chunk_adapter[c];
-        int rk = 0;
-        if (a >= 0) { rk = rank[a]; if (rk < 0) rk = 0; if (rk > 64) rk = 64; }
+        int rk = crk[c];
         w[0] = chunk_len[c];
         w[1] = a;
         w[2] = rk;
@@ -275,6 +296,8 @@ int orc_build_work(const int32_t *chunk_start, const int32_t *chunk_len, const i
             w[16 + j] = v;
         }
     }
+    free(ord);
+    free(crk);
     return ORC_OK;
 }
 

@@ -92,8 +92,21 @@ def test_build_chunks_brute_force(toks, group):
     assert len(cs) <= max(T, 1)
 
 
+def _record_order(ca, rank, P, heavy_first):
+    """Chunk held by every position of the record sequence: chunk order, and for batches of at most 2048 tokens
+    falling rank inside each range of P chunks (one XCD), ties in chunk order (numpy's stable argsort)."""
+    n = len(ca)
+    crk = np.array([min(max(int(rank[a]), 0), 64) if a >= 0 else 0 for a in ca], dtype=np.int64)
+    order = []
+    for lo in range(0, n, max(P, 1)):
+        idx = np.arange(lo, min(lo + P, n))
+        order += list(idx[np.argsort(-crk[idx], kind="stable")] if heavy_first else idx)
+    return order
+
+
 def test_build_work_by_enumeration():
-    """Work records: placement b = (c mod P) * 8 + c // P and contents, checked field by field."""
+    """Work records: position pos of the record sequence sits at b = (pos mod P) * 8 + pos // P; which chunk a
+    position holds (see _record_order) and the contents, checked field by field."""
     rng = np.random.default_rng(8)
     N, T, group, page_rows, n_pages = 9, 45, 4, 8, 40
     rank = rng.choice([8, 16, 24, 64], N).astype(np.int32)
@@ -108,8 +121,16 @@ def test_build_work_by_enumeration():
     assert work.shape == (cap, orc.WORK_WORDS)
     P = -(-len(cs) // 8)
     used = set()
-    for c in range(len(cs)):
-        b = (c % P) * 8 + c // P
+    order = _record_order(ca, rank, P, heavy_first=True)
+    assert sorted(order) == list(range(len(cs)))
+    # heavy first inside a range, and a range keeps its chunks (one XCD, residue pos // P)
+    for pos in range(1, len(order)):
+        if pos % P:
+            ra, rb = (rank[ca[order[k]]] if ca[order[k]] >= 0 else 0 for k in (pos - 1, pos))
+            assert ra >= rb
+    assert all(order[pos] // P == pos // P for pos in range(len(order)))
+    for pos, c in enumerate(order):
+        b = (pos % P) * 8 + pos // P
         used.add(b)
         w = work[b]
         a = int(ca[c])
@@ -124,11 +145,27 @@ def test_build_work_by_enumeration():
             pg = page_tbl[a, j // page_rows]
             want = pg * page_rows + j % page_rows if (j < rank[a] and 0 <= pg < n_pages) else -1
             assert w[16 + j] == want
-    # consecutive chunks share blockIdx mod 8 (one XCD): chunk c sits at residue c // P
-    assert all(((c % P) * 8 + c // P) % 8 == c // P for c in range(len(cs)))
+    # consecutive positions of a range share blockIdx mod 8 (one XCD): position pos sits at residue pos // P
+    assert all(((pos % P) * 8 + pos // P) % 8 == pos // P for pos in range(len(cs)))
     for b in range(cap):
         if b not in used:
             assert work[b, 0] == 0 and work[b, 1] == -1 and np.all(work[b, 2:] == 0)
+
+
+def test_build_work_keeps_chunk_order_beyond_2048_tokens():
+    rng = np.random.default_rng(9)
+    N, T, group, page_rows, n_pages = 40, 2100, 4, 8, 400
+    rank = rng.choice([8, 16, 32, 64], N).astype(np.int32)
+    page_tbl = rng.integers(0, n_pages, (N, 8)).astype(np.int32)
+    scaling = rng.random(N).astype(np.float32)
+    tok = rng.integers(0, N, T).astype(np.int32)
+    perm, ss, sl, sa, nv = orc.build_segments(tok, N)
+    cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, T, group)
+    work = orc.build_work(cs, cl, ca, perm, page_tbl, rank, scaling, page_rows, n_pages, T)
+    P = -(-len(cs) // 8)
+    for c in range(len(cs)):
+        w = work[(c % P) * 8 + c // P]
+        assert w[0] == cl[c] and w[1] == ca[c] and w[4] == perm[cs[c]]
 
 
 def test_sgmv_plan_brute_force():
