@@ -32,8 +32,8 @@ MFMA_PEAK_BF16_TFLOPS = 2500.0      # dense bf16 / fp16 MFMA peak of the device
 # HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
 # profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
 # same runs).  Reported as roofline.traffic only when the run is that same configuration.
-MEASURED_TRAFFIC_C2 = 81.82e6
-MEASURED_TRAFFIC_C4_STEP = 2906.6e6
+MEASURED_TRAFFIC_C2 = 81.78e6
+MEASURED_TRAFFIC_C4_STEP = 2906.7e6
 
 
 def log(*a):
