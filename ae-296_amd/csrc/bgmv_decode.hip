@@ -88,12 +88,16 @@ __global__ __launch_bounds__(NT) void bgmv_kernel(const BgmvArgs p)
         tok[0] = item;
 #pragma unroll
         for (int k = 1; k < G; k++) tok[k] = -1;
-        if (p.tok_adapter) adapter = p.tok_adapter[item];
-        else {
+        if (p.tok_adapter) {
+            // int32 ids: any negative id and any id beyond the pool mean "no adapter" (the row is
+            // defined: kept when accumulating, zeros otherwise), as the work-record path treats them
+            adapter = p.tok_adapter[item];
+            if (adapter < 0 || adapter >= pv.n_adapters) adapter = -1;
+        } else {
+            // int64 ids of the reference-layout call: a bad index leaves the row untouched (-2)
             const long long a64 = p.tok_adapter64[item];
             adapter = (a64 < 0 || a64 >= pv.n_adapters) ? -2 : (int)a64;
         }
-        if (adapter >= pv.n_adapters) adapter = -2;
         r = 0;
         scale = 0.f;
         if (adapter >= 0) {

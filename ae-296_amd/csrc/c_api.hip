@@ -358,7 +358,7 @@ namespace {
 
 constexpr int SG_TM = 64;   // tokens per tile, as in sgmv_prefill.hip
 
-struct SgmvWs { int max_tiles; int ksplit; int ks_cap; size_t off_rec, off_proj, per_proj, off_hi, off_lo, total; };
+struct SgmvWs { int max_tiles; int ksplit; int ks_cap; size_t off_cover, off_rec, off_proj, per_proj, off_hi, off_lo, total; };
 
 // Workspace: the plan (tile list, tile records: depends on T and n_seg only), then per projection the
 // K-split partial sums and the hi / lo halves of their sum.
@@ -377,6 +377,9 @@ SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
     w.ks_cap = n_proj > 1 ? (3 * w.ksplit < 8 ? 3 * w.ksplit : 8) : w.ksplit;
     size_t off = ((size_t)w.max_tiles * 3 + 4) * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
+    w.off_cover = off;                              // int32 [T]: 1 where a token belongs to some segment
+    off += (size_t)T * sizeof(int32_t);
+    off = (off + 255) & ~(size_t)255;
     w.off_rec = off;
     off += (size_t)w.max_tiles * 80 * sizeof(int32_t);
     off = (off + 255) & ~(size_t)255;
@@ -394,6 +397,7 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
     int32_t *ip = reinterpret_cast<int32_t *>(base);
     a.tile_seg = ip; a.tile_tok0 = ip + w.max_tiles; a.tile_ntok = ip + 2 * (size_t)w.max_tiles;
     a.n_tiles = ip + 3 * (size_t)w.max_tiles;
+    a.tok_cover = reinterpret_cast<int32_t *>(base + w.off_cover);
     a.tile_rec = reinterpret_cast<int32_t *>(base + w.off_rec);
     a.max_tiles = w.max_tiles;
     int hin_min = a.pr[0].hin;

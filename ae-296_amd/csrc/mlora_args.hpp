@@ -133,6 +133,7 @@ struct SgmvArgs {
     int32_t *tile_tok0;
     int32_t *tile_ntok;
     int32_t *n_tiles;      // [1]
+    int32_t *tok_cover;    // [T] 1 where a token belongs to a tile (written by the plan): rows of y = delta mode outside are zeroed
     int32_t *tile_rec;     // [max_tiles * TILE_WORDS] per-tile records (layout below)
     int max_tiles;
 };

@@ -128,6 +128,14 @@ __global__ __launch_bounds__(1024) void sgmv_plan_kernel(const SgmvArgs p)
     const int n_tiles = s_carry < p.max_tiles ? s_carry : p.max_tiles;
     if (tid == 0) p.n_tiles[0] = n_tiles;
     __syncthreads();                               // tile_* written above are visible to the whole block
+    // Which tokens belong to a tile at all: y = delta mode must define the rows of the others (zeros).
+    for (int t = tid; t < p.T; t += 1024) p.tok_cover[t] = 0;
+    __syncthreads();
+    for (long long idx = tid; idx < (long long)n_tiles * TM; idx += 1024) {
+        const int tl = (int)(idx / TM), k = (int)(idx - (long long)tl * TM);
+        const int t = p.tile_tok0[tl] + k;
+        if (k < p.tile_ntok[tl] && t >= 0 && t < p.T) p.tok_cover[t] = 1;
+    }
     // Per-tile records: everything a shrink / expand workgroup needs, so that it starts from one load.
     // Headers of up to 1024 tiles at a time go through LDS (one tile per thread), then all threads
     // fill the 80-word records of that batch with one table lookup per row word.
@@ -313,6 +321,15 @@ __global__ __launch_bounds__(256) void sgmv_reduce_kernel(const SgmvArgs p)
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
     if (idx >= (long long)p.T * CPT) return;
     const int t = (int)(idx / CPT), c0 = (int)(idx - (long long)t * CPT) * 8;
+    if (p.tok_cover[t] == 0) {
+        // token outside every segment: no tile touches its row.  y = delta mode defines it as zeros
+        // (the CPT threads of the token share the row); accumulate mode keeps it.
+        if (!p.accumulate) {
+            uint16_t *__restrict__ yrow = static_cast<uint16_t *>(pj.y) + (size_t)t * pj.hout;
+            for (int cc = c0 >> 3; cc < (pj.hout >> 3); cc += CPT) stg16(yrow + (size_t)cc * 8, zero16());
+        }
+        return;
+    }
     float v[8];
 #pragma unroll
     for (int e = 0; e < 8; e++) v[e] = 0.f;

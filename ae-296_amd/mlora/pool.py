@@ -95,6 +95,8 @@ class AdapterPool:
 
     def release(self, slot: int) -> None:
         """Evict the adapter in `slot` (the reference's remove_lora, lora_gpu.py:229-242, without copies)."""
+        if not 0 <= slot < self.n_slots:
+            raise IndexError(f"slot {slot} outside [0, {self.n_slots})")
         need = (int(self.h_rank[slot]) + self.page_rows - 1) // self.page_rows
         self._free.extend(int(p) for p in self.h_page_tbl[slot, :need][::-1])
         self.h_page_tbl[slot, :] = -1
@@ -104,7 +106,15 @@ class AdapterPool:
 
     def move(self, src: int, dst: int) -> None:
         """Re-bind an adapter to another slot (the reference's merge_lora_prefill, lora_gpu.py:202-217,
-        copies every layer's weights; here only the table rows move)."""
+        copies every layer's weights; here only the table rows move).  An adapter already in `dst` is
+        evicted; `src` must hold one and differ from `dst`."""
+        for name, slot in (("src", src), ("dst", dst)):
+            if not 0 <= slot < self.n_slots:
+                raise IndexError(f"{name} slot {slot} outside [0, {self.n_slots})")
+        if src == dst:
+            raise ValueError(f"move({src}, {dst}): source and destination are the same slot")
+        if self.h_rank[src] == 0:
+            raise ValueError(f"move: slot {src} holds no adapter")
         if self.h_rank[dst] != 0:
             self.release(dst)
         self.h_page_tbl[dst] = self.h_page_tbl[src]

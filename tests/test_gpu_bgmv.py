@@ -142,6 +142,34 @@ def test_bgmv_tokens_without_adapter_and_rank_tails():
         assert_close_bits(got_d, oracle_apply(pp, x, tok, None), FP16)
 
 
+def test_bgmv_ids_below_minus_one_and_beyond_the_pool_mean_no_adapter():
+    """An int32 id < -1 or >= n_adapters is "no adapter" in every launch form: the row is kept when
+    accumulating and is zeros in y = delta mode (a caller may hand over torch.empty memory)."""
+    rng = np.random.default_rng(43)
+    N = 5
+    pp = PagedPool(rng, [8, 16, 4, 32, 2], 512, 384, page_rows=8, dtype=FP16)
+    T = 37
+    tok = rng.integers(0, N, T).astype(np.int32)
+    tok[[1, 7, 20]] = -2
+    tok[[3, 8]] = N + 3
+    tok[11] = -1
+    tok[30] = np.iinfo(np.int32).max
+    tok[31] = np.iinfo(np.int32).min
+    none = (tok < 0) | (tok >= N)
+    tok_orc = np.where(none, -1, tok).astype(np.int32)      # the oracle's spelling of "no adapter"
+    x = bits_of(rng.standard_normal((T, 512)).astype(np.float32), FP16)
+    y0 = bits_of(rng.standard_normal((T, 384)).astype(np.float32), FP16)
+    want, want_d = oracle_apply(pp, x, tok_orc, y0), oracle_apply(pp, x, tok_orc, None)
+    for group, fused in ((0, True), (1, True), (4, True), (4, False)):
+        say(f"bgmv out-of-range ids group={group} fused={fused}")
+        got = _run(pp, x, tok, y0, group, fused=fused)
+        assert np.array_equal(got[none], y0[none])
+        assert_close_bits(got, want, FP16)
+        got_d = _run(pp, x, tok, None, group, accumulate=False, fused=fused)      # y starts as NaN
+        assert np.all(got_d[none] == 0)
+        assert_close_bits(got_d, want_d, FP16)
+
+
 def test_bgmv_multi_projection_one_launch():
     """q/k/v share x, o has its own input: one launch, four slabs, each checked against the oracle."""
     rng = np.random.default_rng(43)

@@ -109,8 +109,43 @@ def test_sgmv_segments_without_adapter_and_gaps():
     say("sgmv gaps / adapter-less segment, delta")
     got_d = _run(pp, x, (ss, sl, sa), None, accumulate=False)
     assert np.all(got_d[10:40] == 0)                       # adapter-less segment is defined as zeros
-    covered = tok >= 0
-    assert_close_bits(got_d[covered], oracle_apply(pp, x, tok, None)[covered], FP16)
+    assert np.all(got_d[tok < 0] == 0)                     # ... and so are tokens 0..9 and 124..129, which no segment covers
+    assert_close_bits(got_d, oracle_apply(pp, x, tok, None), FP16)
+
+
+def test_sgmv_delta_defines_rows_outside_every_segment():
+    """y = delta mode over NaN-filled memory: rows between, before and after the segments (given out of
+    order) come back as zeros from the one-projection, the planned and the multi-projection calls."""
+    from mlora import plan_prefill, sgmv, sgmv_multi
+    rng = np.random.default_rng(75)
+    hin, hout = 256, 392
+    pp = PagedPool(rng, [8, 64, 24], hin, hout, page_rows=8, dtype=BF16)
+    ss = np.array([200, 5, 70], np.int32)                  # gaps: 0..4, 69, 135..199, 263..299
+    sl = np.array([63, 64, 65], np.int32)
+    sa = np.array([2, 0, 1], np.int32)
+    T = 300
+    tok = _tok_of(ss, sl, sa, T)
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), BF16)
+    want = oracle_apply(pp, x, tok, None)
+    assert np.all(want[tok < 0] == 0) and (tok < 0).sum() == 108
+    say("sgmv delta with gaps: self-planning call")
+    got = _run(pp, x, (ss, sl, sa), None, accumulate=False)
+    assert np.all(got[tok < 0] == 0)
+    assert_close_bits(got, want, BF16)
+    pool = upload_pool(pp)
+    seg = tuple(torch.from_numpy(a).cuda() for a in (ss, sl, sa))
+    xt = bits_to_torch(x, BF16, "cuda")
+    plan = plan_prefill(*seg, T, pool, n_proj=2)
+    nan = lambda: torch.full((T, hout), float("nan"), dtype=torch.bfloat16, device="cuda")
+    say("sgmv delta with gaps: planned and multi-projection calls")
+    y1, y2, y3 = nan(), nan(), nan()
+    sgmv(y1, xt, pool, 0, "p", accumulate=False, plan=plan)
+    sgmv_multi([y2, y3], [xt, xt], pool, 0, ["p", "p"], plan, accumulate=False)
+    torch.cuda.synchronize()
+    for y in (y1, y2, y3):
+        bits = torch_to_bits(y)
+        assert np.all(bits[tok < 0] == 0)
+        assert_close_bits(bits, want, BF16)
 
 
 def test_sgmv_plan_once_apply_many():

@@ -59,6 +59,28 @@ def test_move_is_a_table_update():
     assert p.free_pages == free
 
 
+def test_move_rejects_bad_arguments_and_evicts_the_destination():
+    p = _pool()
+    p.allocate(0, 32, 1.0)
+    p.allocate(1, 8, 2.0)
+    snap = (p.h_page_tbl.copy(), p.h_rank.copy(), p.free_pages)
+    with pytest.raises(ValueError):
+        p.move(0, 0)                           # would free the adapter's own pages
+    with pytest.raises(ValueError):
+        p.move(3, 1)                           # empty source would silently evict slot 1
+    with pytest.raises(IndexError):
+        p.move(0, 6)
+    with pytest.raises(IndexError):
+        p.move(-1, 2)
+    with pytest.raises(IndexError):
+        p.release(6)
+    assert np.array_equal(p.h_page_tbl, snap[0]) and np.array_equal(p.h_rank, snap[1]) and p.free_pages == snap[2]
+    pages0 = p.h_page_tbl[0].copy()
+    p.move(0, 1)                               # occupied destination: its adapter is evicted, its page returns
+    assert p.free_pages == snap[2] + 1 and p.h_rank[1] == 32 and p.h_rank[0] == 0
+    assert np.array_equal(p.h_page_tbl[1], pages0)
+
+
 def test_load_places_rank_rows_on_the_adapters_pages():
     p = _pool()
     p.allocate(1, 16, 2.0, pages=[7, 2])
