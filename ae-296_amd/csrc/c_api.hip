@@ -4,6 +4,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/mlora.h"
 #include "mlora_args.hpp"
@@ -52,6 +53,37 @@ int check_pool(mlora::PoolView &pv, const int32_t *page_tbl, const int32_t *rank
     pv.n_rows_a = n_pages_a * page_rows; pv.n_rows_b = n_pages_b * page_rows;
     pv.a_dense_stride = 0; pv.b_dense_stride = 0;
     return MLORA_OK;
+}
+
+// Device memory for mlora_bgmv_multi_noalloc: the fp32 intermediate of the two-launch decode form, for
+// callers that cannot allocate.  Every GPU the library runs on holds its own copy of the array at its own
+// address until the process ends; host code only ever uses the per-device address looked up below, never
+// the array's name (which on the host is a stand-in, not a device address).
+constexpr size_t SCRATCH_BYTES = MLORA_NOALLOC_SCRATCH_BYTES;
+__device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+constexpr int SCRATCH_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[SCRATCH_MAX_DEVICES] = {};
+
+// Address of the current device's copy of `scratch` (looked up once per device); nullptr + error text on failure.
+void *scratch_of_current_device()
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { fail(MLORA_ELAUNCH, "hipGetDevice failed: %s", hipGetErrorString(e)); return nullptr; }
+    if (dev < 0 || dev >= SCRATCH_MAX_DEVICES) { fail(MLORA_ERANGE, "device ordinal %d outside [0, %d)", dev, SCRATCH_MAX_DEVICES); return nullptr; }
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            fail(MLORA_ELAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
 }
 
 int check_dims(int hin, int hout)
@@ -233,12 +265,13 @@ int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
     return (int64_t)n_proj * T * ks * mlora::bgmv_split_rank_stride(max_rank) * (int64_t)sizeof(float);
 }
 
-int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+// use_scratch: the two-launch form with the library's own per-device scratch array as its workspace
+static int bgmv_multi_impl(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
                      const void *const *b_rows, const int32_t *hin, const int32_t *hout,
                      const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
                      const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
                      int max_rank, const int32_t *work, int group, void *workspace, int64_t workspace_bytes,
-                     int dtype, int accumulate, void *stream)
+                     bool use_scratch, int dtype, int accumulate, void *stream)
 {
     if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
     if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
@@ -257,7 +290,7 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
     } else if (group != 1) {
         return fail(MLORA_EINVAL, "group must be 1 when work is NULL (got %d)", group);
     }
-    if (workspace && !work) return fail(MLORA_EINVAL, "the two-launch form (workspace given) needs the work records");
+    if ((workspace || use_scratch) && !work) return fail(MLORA_EINVAL, "the two-launch form needs the work records");
     int max_hin = 0, max_hout = 0;
     for (int p = 0; p < n_proj; p++) {
         if (!y[p] || !x[p] || !a_rows[p] || !b_rows[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
@@ -281,6 +314,15 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
         a.items_cap = bound < a.work_cap ? (int)bound : a.work_cap;
     }
     a.T = T; a.n_proj = n_proj; a.accumulate = accumulate ? 1 : 0;
+    if (use_scratch) {
+        const int64_t need = mlora_bgmv_workspace_bytes(n_proj, T, max_hin, max_rank);
+        if (need > (int64_t)SCRATCH_BYTES)
+            return fail(MLORA_ENOSPACE, "this call needs %lld bytes of intermediate, the allocation-free entry point holds %lld "
+                        "(n_proj x T x column slices x rank); use mlora_bgmv_multi with a workspace", (long long)need, (long long)SCRATCH_BYTES);
+        workspace = scratch_of_current_device();
+        if (!workspace) return MLORA_ELAUNCH;
+        workspace_bytes = (int64_t)SCRATCH_BYTES;
+    }
     if (workspace) {
         const int64_t need = mlora_bgmv_workspace_bytes(n_proj, T, max_hin, max_rank);
         if (workspace_bytes < need)
@@ -297,6 +339,30 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const voi
     }
     if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
+}
+
+int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+                     const void *const *b_rows, const int32_t *hin, const int32_t *hout,
+                     const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
+                     const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
+                     int max_rank, const int32_t *work, int group, void *workspace, int64_t workspace_bytes,
+                     int dtype, int accumulate, void *stream)
+{
+    return bgmv_multi_impl(n_proj, y, x, a_rows, b_rows, hin, hout, tok_adapter, T, page_tbl, rank, scaling, n_adapters,
+                           max_pages, page_rows, n_pages, max_rank, work, group, workspace, workspace_bytes, false,
+                           dtype, accumulate, stream);
+}
+
+int mlora_bgmv_multi_noalloc(int n_proj, void *const *y, const void *const *x, const void *const *a_rows,
+                             const void *const *b_rows, const int32_t *hin, const int32_t *hout,
+                             const int32_t *tok_adapter, int T, const int32_t *page_tbl, const int32_t *rank,
+                             const float *scaling, int n_adapters, int max_pages, int page_rows, int64_t n_pages,
+                             int max_rank, const int32_t *work, int group, int dtype, int accumulate, void *stream)
+{
+    if (!work) return fail(MLORA_EINVAL, "mlora_bgmv_multi_noalloc needs the work records of mlora_pool_gather");
+    return bgmv_multi_impl(n_proj, y, x, a_rows, b_rows, hin, hout, tok_adapter, T, page_tbl, rank, scaling, n_adapters,
+                           max_pages, page_rows, n_pages, max_rank, work, group, nullptr, 0, true,
+                           dtype, accumulate, stream);
 }
 
 int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows, const int32_t *tok_adapter,

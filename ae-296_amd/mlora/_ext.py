@@ -24,6 +24,7 @@ GATHER_MAX_T = 8192
 CNT_NSEG, CNT_NVALID, CNT_NCHUNK, CNT_BAD, CNT_WORDS = 0, 1, 2, 3, 8
 WORK_WORDS = 80
 SCATTER_MAX_JOBS = 16
+NOALLOC_SCRATCH_BYTES = 16 << 20    # MLORA_NOALLOC_SCRATCH_BYTES
 
 
 def work_cap(T: int) -> int:
@@ -46,6 +47,8 @@ SIGNATURES = {
     "mlora_bgmv_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
                                 _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),
+    "mlora_bgmv_multi_noalloc": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
+                                        _i64, _i32, _vp, _i32, _i32, _i32, _vp]),
     "mlora_bgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i64,
                           _i32, _i32, _i32, _vp]),
     "mlora_bgmv_reflayout": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),

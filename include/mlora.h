@@ -183,6 +183,30 @@ int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
                      void *workspace, int64_t workspace_bytes,
                      int dtype, int accumulate, void *stream);
 
+/*
+ * mlora_bgmv_multi in its two-launch form with no workspace argument and no allocation anywhere on its
+ * path.  No counterpart in the reference: it is for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc) and so cannot provide the
+ * workspace of the call above.  The fp32 intermediate lives in a file-scope device array of
+ * MLORA_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends; a call that
+ * needs more (mlora_bgmv_workspace_bytes(n_proj, T, max hin, max_rank): n_proj x T x column slices x rank
+ * stride x 4 bytes) returns MLORA_ENOSPACE.  `work` (the records of mlora_pool_gather) is required.  Results
+ * are those of mlora_bgmv_multi with a workspace, bit for bit.  The array keeps the previous call's contents;
+ * nothing in it has to start at zero (the shrink launch writes every value the expand launch reads).  All
+ * calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race; order
+ * them on one stream.  The array's device address is looked up on the first call on each device (a runtime
+ * query, no allocation): make that first call outside graph capture.
+ */
+#define MLORA_NOALLOC_SCRATCH_BYTES (16u << 20)
+int mlora_bgmv_multi_noalloc(int n_proj, void *const *y, const void *const *x,
+                             const void *const *a_rows, const void *const *b_rows,
+                             const int32_t *hin, const int32_t *hout,
+                             const int32_t *tok_adapter, int T,
+                             const int32_t *page_tbl, const int32_t *rank, const float *scaling,
+                             int n_adapters, int max_pages, int page_rows, int64_t n_pages, int max_rank,
+                             const int32_t *work, int group,
+                             int dtype, int accumulate, void *stream);
+
 /* One projection, one token per work item: the plain form of the call above. */
 int mlora_bgmv(void *y, const void *x, const void *a_rows, const void *b_rows,
                const int32_t *tok_adapter,

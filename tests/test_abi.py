@@ -71,6 +71,18 @@ def test_validation_errors_without_gpu():
         _ext.check(bgmv(dtype=7))
     assert e.value.code == _ext.MLORA_EDTYPE
 
+    # the allocation-free form: needs work records, and refuses a batch whose intermediate exceeds its fixed array
+    def noalloc(T=4, work=one, n_proj=1, hin=H, max_rank=64):
+        return lib.mlora_bgmv_multi_noalloc(n_proj, P, P, P, P, hin, H, one, T, one, one, one, 4, 8, 8, 10, max_rank,
+                                            work, 4, 0, 1, None)
+    assert noalloc(work=None) == _ext.MLORA_EINVAL
+    assert b"work records" in lib.mlora_last_error()
+    big = (C.c_int32 * 8)(*([11008] * 8))
+    assert lib.mlora_bgmv_workspace_bytes(8, 8192, 11008, 64) > _ext.NOALLOC_SCRATCH_BYTES
+    assert noalloc(T=8192, n_proj=8, hin=big) == _ext.MLORA_ENOSPACE
+    assert b"allocation-free" in lib.mlora_last_error()
+    assert noalloc(T=0) == _ext.MLORA_OK
+
     rc = lib.mlora_pool_gather(one, 9000, one, one, one, 4, 8, 8, 10, None, None, None, one, one, one, one, one, one, one, 4, one, one, None)
     assert rc == _ext.MLORA_ERANGE                     # more tokens than one gather call groups
     rc = lib.mlora_pool_gather(one, 10, one, one, one, 4, 8, 8, 10, None, None, None, one, None, one, one, one, one, one, 4, one, None, None)
