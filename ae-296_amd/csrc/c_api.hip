@@ -177,6 +177,16 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
     return MLORA_OK;
 }
 
+int mlora_probe_stream(void *buf, int64_t bytes, int mode, void *stream)
+{
+    if (bytes < 0 || (mode != 0 && mode != 1)) return fail(MLORA_EINVAL, "bytes must be >= 0 and mode 0 (read) or 1 (read-modify-write)");
+    if (bytes == 0) return MLORA_OK;
+    if (!buf || !aligned16(buf)) return fail(MLORA_EALIGN, "buf must be a 16-byte aligned device pointer");
+    const int rc = mlora::launch_stream_probe(buf, bytes, mode, nullptr, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "probe launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
 int mlora_host_alloc(int64_t bytes, void **host_ptr, void **dev_ptr)
 {
     if (bytes <= 0 || !host_ptr || !dev_ptr) return fail(MLORA_EINVAL, "bytes must be positive and the out pointers non-NULL");

@@ -1,0 +1,45 @@
+// Streaming probe: what a plain pass over device memory reaches on this device, measured by the benchmark in
+// the same run as the LoRA kernels so that their figures can be read against the box's own ceiling (which
+// differs from box to box and lies well under the published HBM peak).  MODE 0 reads every 16 bytes once with
+// the nontemporal loads the LoRA kernels use; MODE 1 reads, changes and writes back in place (the access
+// pattern of an accumulate-into-y expand).  No counterpart in the reference.
+#include "mlora_args.hpp"
+#include "mlora_dev.hpp"
+
+namespace mlora {
+
+template <int MODE>
+__global__ __launch_bounds__(256) void stream_probe_kernel(uint4 *__restrict__ p, long long n16, unsigned *__restrict__ sink)
+{
+    constexpr int U = 8;                                   // 16-byte loads in flight per thread
+    const long long stride = (long long)gridDim.x * 256 * U;
+    unsigned acc = 0;
+    for (long long i = (long long)blockIdx.x * 256 * U + threadIdx.x; i < n16; i += stride) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const long long idx = i + (long long)u * 256;
+            v[u] = idx < n16 ? ldg16_stream(p + idx) : zero16();
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const long long idx = i + (long long)u * 256;
+            if constexpr (MODE == 0) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+            else if (idx < n16) { v[u].x += 1u; stg16_stream(p + idx, v[u]); }
+        }
+    }
+    if (MODE == 0 && acc == 0x9e3779b9u && sink) sink[0] = acc;      // keeps the loads alive; practically never taken
+}
+
+int launch_stream_probe(void *p, long long bytes, int mode, unsigned *sink, hipStream_t s)
+{
+    const long long n16 = bytes / 16;
+    if (n16 <= 0) return 0;
+    long long blocks = (n16 + 256 * 8 - 1) / (256 * 8);
+    if (blocks > 2048) blocks = 2048;                      // eight workgroups per compute unit, each striding over the buffer
+    if (mode == 0) hipLaunchKernelGGL(stream_probe_kernel<0>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<uint4 *>(p), n16, sink);
+    else hipLaunchKernelGGL(stream_probe_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<uint4 *>(p), n16, sink);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mlora

@@ -4,7 +4,7 @@ Host layer in Python over ``libmlora_hip.so`` (hand-written gfx950 kernels behin
 ``include/mlora.h``).  Importing the package does not load the extension; the first call does,
 and raises if it has not been built.
 """
-from . import _ext
+from . import _ext, cpu_ops
 from ._ext import MloraError
 from .loader import AdapterLoader, HostAdapter, LoadTicket, layer_order
 from .lora_cpu import Lora_CPU
@@ -14,4 +14,4 @@ from .ops import (DecodePlan, PrefillPlan, add_lora_bgmv, bgmv, gemm_lora, lora_
 from .pool import AdapterPool
 
 __all__ = ["AdapterLoader", "AdapterPool", "HostAdapter", "LoadTicket", "layer_order", "DecodePlan", "Lora_CPU", "Lora_GPU", "MloraError", "add_lora_bgmv", "bgmv", "gemm_lora", "lora_apply",
-           "lora_prefill_ref", "plan_decode", "plan_prefill", "PrefillPlan", "sgmv", "sgmv_multi", "sgmv_workspace", "_ext"]
+           "lora_prefill_ref", "plan_decode", "plan_prefill", "PrefillPlan", "sgmv", "sgmv_multi", "sgmv_workspace", "_ext", "cpu_ops"]

@@ -40,6 +40,7 @@ SIGNATURES = {
     "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
     "mlora_pool_scatter": (_i32, [_i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i32, _vp]),
+    "mlora_probe_stream": (_i32, [_vp, _i64, _i32, _vp]),
     "mlora_host_alloc": (_i32, [_i64, _vp, _vp]),
     "mlora_host_free": (_i32, [_vp]),
     "mlora_assist_export": (_i32, [_vp, _i32, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),

@@ -2,10 +2,10 @@
 the CPU-assisted path, on which host workers compute the LoRA delta of the early layers while an
 adapter is still being loaded into the pool.
 
-Only the transport is here -- shipping hidden states to the workers, waking them, and bringing their
-results back.  The arithmetic stays with the workers (the reference's ``lora_cpu/lora_shm_op/app.py``
-processes, or any host code that follows the protocol below); nothing in this package computes a
-LoRA delta on the CPU.
+This class is the transport -- shipping hidden states to the workers, waking them, and bringing their
+results back.  The workers are any host code that follows the protocol below: the reference's
+``lora_cpu/lora_shm_op/app.py`` processes, or the in-process thread pool of ``libmlora_cpu.so``
+(``start_workers``), which computes the chunks with the package's own CPU kernel (``cpu_ops.py``).
 
 Protocol (the reference's, ``lora_cpu.py:138-276`` and ``app.py:102-143``, with its result placement
 restated from the arithmetic, because worker and collector of the reference only agree when a request
@@ -30,7 +30,7 @@ from typing import List, Optional, Tuple
 import numpy as np
 import torch
 
-from . import _ext
+from . import _ext, cpu_ops
 
 PROMPT_MAX_LENGTH = 256          # tokens per request slot (lora_cpu.py:14)
 SIGNAL_BASE, SIGNAL_STRIDE = 2, 200   # codes 2.., 202.., 402.. (lora_cpu.py:181-185, app.py:110-128)
@@ -85,8 +85,34 @@ class Lora_CPU:
         self.np_signal, self.np_tkn_len = self._signal.array, self._tkn_len.array
         self.active_cpu = 0
         self._dtype = torch.float16
+        self._workers = None
+        self._worker_pool = None
+
+    # ------------------------------------------------------------------ in-process workers
+    def start_workers(self, down, up, n_threads: int, slot_adapter=None) -> None:
+        """Serve the slots from a pool of `n_threads` host threads inside this process (instead of the
+        reference's one pinned process per request chunk and projection, ``runServerCPULoRA.py:74-90``):
+        ``down[q] [N, H, r]`` / ``up[q] [N, r, H]`` (fp32 or binary16) are the q, k, v adapters,
+        ``slot_adapter [lora_num]`` the adapter of the request in each slot (None: adapter 0).  fp16 only."""
+        if self._workers is not None:
+            raise RuntimeError("workers are already running")
+        self._worker_pool = cpu_ops.CpuLoraPool(n_threads)
+        self._workers = cpu_ops.AssistWorkers(self._worker_pool, self.np_x, self.np_out, self.np_signal, self.np_tkn_len,
+                                              self.cpu_capacity, down, up, slot_adapter, SIGNAL_BASE, SIGNAL_STRIDE)
+
+    def stop_workers(self):
+        """Stop the in-process workers; returns (chunks served, codes rejected)."""
+        out = (0, 0)
+        if self._workers is not None:
+            out = self._workers.stop()
+            self._workers = None
+        if self._worker_pool is not None:
+            self._worker_pool.close()
+            self._worker_pool = None
+        return out
 
     def close(self):
+        self.stop_workers()
         for m in [self._x, self._signal, self._tkn_len] + self._out:
             m.free()
 

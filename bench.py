@@ -1,23 +1,32 @@
 #!/usr/bin/env python3
-"""Benchmark of the multi-LoRA decode hot path on one MI355X.
+"""Benchmark of the multi-LoRA apply hot path on one MI355X.
 
-Workload (the configuration the metric is quoted on): decode BGMV over the Llama-7B attention
-projections q/k/v/o (4096 -> 4096 each), 256 decode tokens, 64 rank-16 fp16 adapters in one paged
-pool, adapter per token ~ Zipf(1.0), scaling 2.0.  One step = one decode step's LoRA work: the
-adapter-pool gather once, then for each of the 32 layers one BGMV call (a shrink launch and an
-expand launch, or one fused launch with --fused) covering that layer's q, k, v (shared input) and
-o (own input), accumulating into the base projection outputs.
-Every layer has its own pool slabs, inputs and outputs (about 2.4 GB in all), so a step streams
-from HBM rather than from the 256 MB last-level cache.
+Default run (`python bench.py --gpus 1 --steps K --warmup W`): one JSON line whose headline is the largest
+configuration that fits one GPU -- config 5: one decode step of a Llama-2-7B-shaped LoRA path, 32 layers x 7
+projections, 1000 rank-32 adapters resident in a paged pool (about 160 GB), 512 decode tokens Zipf(1.1) through
+BGMV plus 8 prefill segments of 512 tokens through SGMV in the same step -- and whose `legs` object carries the
+other configurations, each timed in the same process on the same device:
 
-Prints one JSON line: throughput in token-projections/s, the HBM roofline of the BGMV call
-(algorithmic bytes / measured duration of one layer's launches) and the CPU baseline (the CPU-assisted path's
-arithmetic timed on the host cores).
+    c1  single LoRA-delta op (the CPU reference's case)        c4  prefill SGMV, Llama-13B shapes, bf16
+    c2  decode BGMV, 256 tokens, 64 rank-16 adapters           f1  base projection + LoRA in one pass (c4 batch)
+    c3  heterogeneous-rank decode BGMV, 7 projections          reflayout  the reference's own pool layout and call
+    maf_trace  a continuous-batching decode sequence driven by the reference's arrival trace and popularity vector
+
+One step of a decode workload = the adapter-pool gather once, then for each layer one BGMV call covering that
+layer's projections, accumulating into the base projection outputs; every layer has its own slabs, inputs and
+outputs so that a step streams from HBM, not from the 256 MB last-level cache; steps are replayed from a HIP
+graph.  `--workload NAME` runs one workload alone and prints its full line.
+
+Every line carries `roofline` (algorithmic bytes or flops of the dominant launches / their measured duration,
+HIP events on the launch stream) and the headline carries `cpu_baseline` (the CPU-assisted path's arithmetic on
+the host cores, through the package's own CPU library) and `stream_ceiling` (what a plain streaming pass reaches
+on this device in this run).
 """
 from __future__ import annotations
 
 import argparse
 import json
+import math
 import os
 import sys
 import time
@@ -29,15 +38,42 @@ for _p in (ROOT, os.path.join(ROOT, "ae-296_amd")):
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_BF16_TFLOPS = 2500.0      # dense bf16 / fp16 MFMA peak of the device
-# HBM bytes per BGMV call (shrink + expand launch) of the default workload, from the two counter runs summarised in
-# profiles/bgmv_c2_bench.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 256 MiB copy in the
-# same runs).  Reported as roofline.traffic only when the run is that same configuration.
-MEASURED_TRAFFIC_C2 = 81.78e6
-MEASURED_TRAFFIC_C4_STEP = 2906.7e6
+MIN_LEG_MS = 100.0                  # every leg is repeated until its timed region is at least this long
+
+# HBM bytes per launch from rocprofv3 counter runs (FETCH_SIZE and WRITE_SIZE, scaled by a copy of known size):
+# the figures live in the committed profile summaries, one `key: value` line each, and are read from there.
+TRAFFIC_SOURCE = {
+    "c2": ("profiles/bgmv_c2_bench.txt", "hbm_bytes_per_decode_call"),
+    "c4": ("profiles/sgmv_c4_bench.txt", "hbm_bytes_per_step"),
+    "c5": ("profiles/mixed_c5_bench.txt", "hbm_bytes_per_decode_call"),
+}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def profile_value(rel_path, key):
+    """`key: <number>` from a profile summary under profiles/ (None when the file or the line is absent)."""
+    try:
+        with open(os.path.join(ROOT, rel_path)) as f:
+            for line in f:
+                s = line.strip()
+                if s.startswith(key + ":"):
+                    return float(s.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def traffic_of(workload, applies=True):
+    """(traffic, traffic_source) of a roofline object."""
+    if workload not in TRAFFIC_SOURCE or not applies:
+        return None, None
+    path, key = TRAFFIC_SOURCE[workload]
+    v = profile_value(path, key)
+    return v, (f"{path} ({key}; rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload, not this run)"
+               if v is not None else f"{path} has no {key} line")
 
 
 def algorithmic_bytes(T, projs, ranks_of_unique, elt=2):
@@ -48,58 +84,187 @@ def algorithmic_bytes(T, projs, ranks_of_unique, elt=2):
     return total
 
 
-def cpu_baseline(seconds=12.0):
-    """The reference's CPU-assisted LoRA arithmetic (x.float() @ down @ up -> half, one task per
-    request chunk) on config 1: 32 tokens, 8 rank-16 adapters, 4096 -> 4096, timed on the host cores."""
+# ---------------------------------------------------------------------------------------------- timing
+def percentiles(xs):
+    s = sorted(xs)
+    pick = lambda q: s[min(len(s) - 1, max(0, int(round(q * (len(s) - 1)))))]
+    return {"p10": pick(0.10), "p50": pick(0.50), "p90": pick(0.90)}
+
+
+def timed(run, reps, warmup):
+    """`reps` calls of run() after `warmup` untimed ones, an event after every call on the stream the kernels
+    run on.  Returns mean ms per call (first event to last) and the spread of the per-call times."""
+    import torch
+    for _ in range(warmup):
+        run()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(reps):
+        run()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    total = ev[0].elapsed_time(ev[reps])
+    per = [ev[i].elapsed_time(ev[i + 1]) for i in range(reps)]
+    out = {"ms": total / reps, "reps": reps, "timed_ms": total, "wall_s": wall}
+    out.update(percentiles(per))
+    return out
+
+
+def reps_for(run, steps, min_ms=MIN_LEG_MS, cap=5000):
+    """Repetitions that make the timed region at least min_ms long (never fewer than `steps`)."""
+    import torch
+    run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        run()
+    torch.cuda.synchronize()
+    est_ms = max((time.perf_counter() - t0) * 1e3 / 3, 1e-3)
+    return int(min(cap, max(steps, math.ceil(min_ms / est_ms))))
+
+
+def graph_of(fn, enabled=True):
+    import torch
+    if not enabled:
+        return fn
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    return g.replay
+
+
+def stream_ceiling(dev):
+    """What one plain streaming launch reaches on this device now: nontemporal read of 84 MB and of 1 GB, and an
+    in-place read-modify-write of 94 MB and of 1 GB (bytes read + written), rotating over 3 GB so that nothing
+    is served by the last-level cache."""
+    import torch
+
+    import mlora
+    lib = mlora._ext.lib()
+    buf = torch.empty(3 << 30, dtype=torch.uint8, device=dev)
+    buf.zero_()
+    out = {}
+    for name, nbytes, mode in (("read_84MB", 84 << 20, 0), ("read_1GB", 1 << 30, 0), ("rmw_94MB", 47 << 20, 1), ("rmw_1GB", 512 << 20, 1)):
+        n_regions = (3 << 30) // nbytes
+        state = {"i": 0}
+
+        def run():
+            off = (state["i"] % n_regions) * nbytes
+            state["i"] += 1
+            mlora._ext.check(lib.mlora_probe_stream(buf.data_ptr() + off, nbytes, mode, mlora._ext.current_stream_ptr()))
+
+        # launches back to back between two events (an event per launch would add its own gap to a 13 us launch);
+        # best of five such blocks
+        n = max(20, min(200, (12 << 30) // nbytes))
+        for _ in range(3):
+            run()
+        best = None
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                run()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / n
+            best = ms if best is None or ms < best else best
+        moved = nbytes * (2 if mode else 1)
+        out[name] = {"GBs": moved / (best * 1e-3) / 1e9, "us": best * 1e3, "frac_of_peak": moved / (best * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    del buf
+    torch.cuda.empty_cache()
+    out["note"] = "mean of back-to-back launches (best of five blocks), HIP events; rmw counts bytes read + bytes written"
+    return out
+
+
+# ---------------------------------------------------------------------------------------------- CPU baseline
+def host_cores():
+    phys = set()
+    try:
+        pid = cid = None
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("physical id"):
+                    pid = line.split(":")[1].strip()
+                elif line.startswith("core id"):
+                    cid = line.split(":")[1].strip()
+                elif not line.strip():
+                    if pid is not None and cid is not None:
+                        phys.add((pid, cid))
+                    pid = cid = None
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"os_cpu_count": os.cpu_count(), "physical_cores": len(phys) or None, "usable_by_this_process": usable}
+
+
+def cpu_baseline(seconds=3.0):
+    """The reference's CPU-assisted LoRA arithmetic (`x.float() @ down @ up -> half`, lora_cpu/lora_shm_op/app.py:136-141,
+    one task per request chunk as lora_cpu.py:150-151 shards it) on config 1 -- 32 tokens, 8 rank-16 adapters,
+    4096 -> 4096, fp32 weights -- through the package's CPU library (libmlora_cpu.so) on 1 thread and on every
+    usable core, and through torch (the library the reference's workers call) on 1 thread and on all."""
     import numpy as np
-    from oracle import oracle as orc
+    import torch
+
+    from mlora import cpu_ops
     rng = np.random.default_rng(1001)
     T, N, r, H = 32, 8, 16, 4096
     down = (rng.standard_normal((N, H, r)) * 0.02).astype(np.float32)
     up = (rng.standard_normal((N, r, H)) * 0.02).astype(np.float32)
     x = rng.standard_normal((T, H)).astype(np.float16).view(np.uint16)
-    req_adapter = rng.integers(0, N, T).astype(np.int32)
-    cores = max(1, min(16, os.cpu_count() or 1))
-    pool = orc.CpuLoraPool(cores)                                       # persistent workers, as the reference's are
+    tok = rng.integers(0, N, T).astype(np.int32)
+    host = host_cores()
+    all_threads = max(1, min(host["usable_by_this_process"], 64))
     out_buf = np.empty((T, H), np.uint16)
-    pool.run(x, down, up, req_adapter, 1, 8, out_buf)                  # warm-up
-    n, t0 = 0, time.perf_counter()
-    while time.perf_counter() - t0 < seconds:
-        pool.run(x, down, up, req_adapter, 1, 8, out_buf)
-        n += 1
-    dt = time.perf_counter() - t0
-    pool.close()
-    out = {"value": T * n / dt, "unit": "token-projections/s", "cores": cores, "kind": "port",
-           "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights), {n} repetitions "
-                     f"in {dt:.1f} s, one task per token over {cores} persistent worker threads"}
-    # The same expression through the library the reference's workers call (torch CPU matmul, one thread per
-    # worker as shared_tensor.py:35 / runServerCPULoRA.py:83 pin it): one request per call, a few seconds.
-    import torch
-    prev = torch.get_num_threads()
-    try:
-        torch.set_num_threads(1)
-        xt = torch.from_numpy(x.view(np.float16).copy())
-        dn, upt = torch.from_numpy(down), torch.from_numpy(up)
-        m, t1 = 0, time.perf_counter()
-        while time.perf_counter() - t1 < 3.0:
-            for t in range(T):
-                a = int(req_adapter[t])
-                (xt[t:t + 1].float() @ dn[a] @ upt[a]).half()
-            m += 1
-        d1 = time.perf_counter() - t1
-        out["torch_cpu_one_thread"] = {"value": T * m / d1, "unit": "token-projections/s", "cores": 1,
-                                       "sample": f"x.float() @ down @ up -> half per request with torch on one thread, "
-                                                 f"{m} repetitions in {d1:.1f} s"}
-    finally:
-        torch.set_num_threads(prev)
-    return out
+
+    def port(n_threads):
+        pool = cpu_ops.CpuLoraPool(n_threads)
+        try:
+            cpu_ops.cpu_lora(x, down, up, tok, out=out_buf, tokens_per_task=8, pool=pool)
+            n, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < seconds:
+                cpu_ops.cpu_lora(x, down, up, tok, out=out_buf, tokens_per_task=8, pool=pool)
+                n += 1
+            dt = time.perf_counter() - t0
+        finally:
+            pool.close()
+        return {"value": T * n / dt, "unit": "token-projections/s", "threads": n_threads, "repetitions": n, "seconds": dt}
+
+    def torch_ref(n_threads):
+        prev = torch.get_num_threads()
+        try:
+            torch.set_num_threads(n_threads)
+            xt = torch.from_numpy(x.view(np.float16).copy())
+            dn, upt = torch.from_numpy(down), torch.from_numpy(up)
+            m, t1 = 0, time.perf_counter()
+            while time.perf_counter() - t1 < seconds:
+                for t in range(T):
+                    a = int(tok[t])
+                    (xt[t:t + 1].float() @ dn[a] @ upt[a]).half()
+                m += 1
+            d1 = time.perf_counter() - t1
+        finally:
+            torch.set_num_threads(prev)
+        return {"value": T * m / d1, "unit": "token-projections/s", "threads": n_threads, "repetitions": m, "seconds": d1}
+
+    p1, pall = port(1), port(all_threads)
+    t1, tall = torch_ref(1), torch_ref(all_threads)
+    return {"value": pall["value"], "unit": "token-projections/s", "cores": all_threads, "kind": "port",
+            "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights, one task per token) repeated for "
+                      f"{seconds:.0f} s per figure: libmlora_cpu.so on 1 and on {all_threads} persistent worker threads, torch "
+                      f"(x.float() @ down @ up -> half per request) on 1 and on {all_threads} threads",
+            "host": host, "port_one_thread": p1, "port_all_threads": pall, "torch_one_thread": t1, "torch_all_threads": tall}
 
 
 def cpu_baseline_prefill(with_base, seconds=10.0):
-    """The oracle (scalar C, one core) on a bounded sample of the config-4 prefill: one segment (128 tokens, or
+    """The checker's scalar C on one core over a bounded sample of the config-4 prefill: one segment (128 tokens, or
     32 with the base product) on one rank-64 adapter, q projection 5120 -> 5120, bf16 -- the LoRA delta added
-    into y (`with_base` False, the SGMV step) or y = x W + delta (`with_base` True).  Reported in the GPU
-    line's unit (TFLOP/s)."""
+    into y (`with_base` False, the SGMV step) or y = x W + delta (`with_base` True), in TFLOP/s."""
     import numpy as np
     from oracle import oracle as orc
     rng = np.random.default_rng(1004)
@@ -131,10 +296,8 @@ def cpu_baseline_prefill(with_base, seconds=10.0):
                       f"{', with the base product' if with_base else ''}: {n} repetitions in {dt:.1f} s on one core"}
 
 
-def bench_c4(args, dev):
-    """Prefill SGMV, config 4: Llama-13B shapes (hidden 5120, MLP 13824), 16 requests with prompt lengths
-    U[128, 1024], each bound to one of 32 rank-64 adapters, bf16, tokens packed per request.  One step =
-    the seven projections of one layer (q, k, v, o, gate, up, down), each one mlora_sgmv call."""
+# ---------------------------------------------------------------------------------------------- prefill workloads
+def _c4_batch(dev, with_weights):
     import numpy as np
     import torch
 
@@ -148,7 +311,7 @@ def bench_c4(args, dev):
     projections = workloads.LLAMA13B_ALL
     pool = mlora.AdapterPool(1, projections, 32, 32 * 8, page_rows=8, max_rank=64, dtype=torch.bfloat16, device=dev)
     workloads.fill_pool(pool, np.full(32, 64, np.int32), np.full(32, 0.5, np.float32), rng, seed=1004)
-    ss, sl, sa = (torch.from_numpy(a).to(dev) for a in (starts, lens, adapters))
+    seg = tuple(torch.from_numpy(a).to(dev) for a in (starts, lens, adapters))
     gen = torch.Generator(device=dev)
     gen.manual_seed(4004)
     x = {h: torch.randn(T, h, device=dev, generator=gen).bfloat16() for h in (5120, 13824)}
@@ -157,84 +320,76 @@ def bench_c4(args, dev):
     x_o = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
     x_ffn = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
     x_in = {"q": x[5120], "k": x[5120], "v": x[5120], "o": x_o, "gate": x_ffn, "up": x_ffn, "down": x[13824]}
+    w = None
+    if with_weights:
+        w = {p: (torch.randn(projections[p], device=dev, generator=gen) / projections[p][0] ** 0.5).bfloat16() for p in projections}
     ws = mlora.sgmv_workspace(T, 16, dev, n_proj=len(projections))
-    names = list(projections)
+    return dict(T=T, projections=projections, pool=pool, seg=seg, adapters=adapters, x=x, y=y, x_in=x_in, w=w, ws=ws,
+                names=list(projections))
+
+
+def bench_c4(args, dev, steps, warmup, min_ms=0.0, cpu=True):
+    """Prefill SGMV, config 4: Llama-13B shapes (hidden 5120, MLP 13824), 16 requests with prompt lengths
+    U[128, 1024], each bound to one of 32 rank-64 adapters, bf16, tokens packed per request.  One step =
+    the plan once, then the seven projections of one layer (q, k, v, o, gate, up, down) in one call."""
+    import numpy as np
+
+    import mlora
+    b = _c4_batch(dev, False)
+    T, projections, pool, names, y, x, x_in = b["T"], b["projections"], b["pool"], b["names"], b["y"], b["x"], b["x_in"]
 
     def step():
-        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)      # once per batch, shared by the projections
-        if args.fused:                                                     # one call per projection (3 launches each)
+        plan = mlora.plan_prefill(*b["seg"], T, pool, workspace=b["ws"])      # once per batch, shared by the projections
+        if args.fused:                                                        # one call per projection (3 launches each)
             for p, (hin, hout) in projections.items():
                 mlora.sgmv(y[p], x[hin], pool, 0, p, accumulate=True, plan=plan)
-        else:                                                              # all seven in one call (3 launches)
+        else:                                                                 # all seven in one call (3 launches)
             mlora.sgmv_multi([y[p] for p in names], [x_in[p] for p in names], pool, 0, names, plan)
 
-    step()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(args.steps):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    ms_per_step = e0.elapsed_time(e1) / args.steps
+    reps = reps_for(step, steps, min_ms) if min_ms else steps
+    t = timed(step, reps, warmup)
+    ms_per_step = t["ms"]
     flops = sum(2.0 * 64 * (hin + hout) * T for hin, hout in projections.values())
-    uniq = np.unique(adapters)
+    uniq = np.unique(b["adapters"])
     alg = sum(T * hin * 2 + 2 * T * hout * 2 + len(uniq) * 64 * (hin + hout) * 2 + 4 * T + 12 * 16
               for hin, hout in projections.values())
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     gbs = alg / (ms_per_step * 1e-3) / 1e9
-    out = {"metric": "SGMV prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
-           "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
-           "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-           "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
-                                  "32 rank-64 adapters, bf16", "tokens": T, "segments": 16},
-           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                        "traffic": None if args.fused else MEASURED_TRAFFIC_C4_STEP, "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
-                                  "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
-                        "algorithmic_bytes_per_step": alg, "mfma_tflops": tflops, "mfma_frac_of_2500": tflops / 2500.0},
-           "cpu_baseline": None if args.no_cpu else cpu_baseline_prefill(False)}
-    print(json.dumps(out), flush=True)
+    traffic, src = traffic_of("c4", not args.fused)
+    return {"metric": "SGMV prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": reps,
+            "warmup": warmup, "ms_per_step": ms_per_step, "ms_per_step_spread": {k: t[k] for k in ("p10", "p50", "p90")},
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "config 4: prefill SGMV, Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
+                                   "32 rank-64 adapters, bf16", "tokens": T, "segments": 16,
+                       "form": "one call per projection" if args.fused else "one call over the 7 projections"},
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                         "traffic": traffic, "traffic_source": src,
+                         "kernel": "sgmv plan (once) + 7 x (shrink, reduce, expand)" if args.fused else
+                                   "sgmv plan (once) + one shrink, reduce and expand launch over the 7 projections",
+                         "algorithmic_bytes_per_step": alg, "flops_per_step": flops, "mfma_tflops": tflops,
+                         "mfma_frac": tflops / MFMA_PEAK_BF16_TFLOPS,
+                         "mfma_frac_ceiling": (flops / alg) / (MFMA_PEAK_BF16_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9))},
+            "cpu_baseline": cpu_baseline_prefill(False) if cpu else None}
 
 
-def bench_f1(args, dev):
+def bench_f1(args, dev, steps, warmup, min_ms=0.0, cpu=True):
     """Base projection + LoRA in one pass on the config-4 batch (Llama-13B shapes, 16 requests U[128, 1024],
     32 rank-64 adapters, bf16): one step = q, k, v, o, gate, up, down of one layer, y = x W + delta, as one
     mlora_gemm_lora_planned call (shrink, scaled reduce, one GEMM launch).  The same step as the reference runs
     it -- library GEMM per projection, then the SGMV kernels adding the delta -- is timed beside it."""
-    import numpy as np
     import torch
 
     import mlora
-    from mlora import workloads
-    rng = np.random.default_rng(1004)
-    lens = rng.integers(128, 1025, 16).astype(np.int32)
-    adapters = rng.integers(0, 32, 16).astype(np.int32)
-    starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
-    T = int(lens.sum())
-    projections = workloads.LLAMA13B_ALL
-    pool = mlora.AdapterPool(1, projections, 32, 32 * 8, page_rows=8, max_rank=64, dtype=torch.bfloat16, device=dev)
-    workloads.fill_pool(pool, np.full(32, 64, np.int32), np.full(32, 0.5, np.float32), rng, seed=1004)
-    ss, sl, sa = (torch.from_numpy(a).to(dev) for a in (starts, lens, adapters))
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(4004)
-    x = {h: torch.randn(T, h, device=dev, generator=gen).bfloat16() for h in (5120, 13824)}
-    x_o = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
-    x_ffn = torch.randn(T, 5120, device=dev, generator=gen).bfloat16()
-    x_in = {"q": x[5120], "k": x[5120], "v": x[5120], "o": x_o, "gate": x_ffn, "up": x_ffn, "down": x[13824]}
-    names = list(projections)
-    w = {p: (torch.randn(projections[p], device=dev, generator=gen) / projections[p][0] ** 0.5).bfloat16() for p in names}
+    b = _c4_batch(dev, True)
+    T, projections, pool, names, x_in, w = b["T"], b["projections"], b["pool"], b["names"], b["x_in"], b["w"]
     y = {p: torch.empty(T, projections[p][1], device=dev, dtype=torch.bfloat16) for p in names}
-    ws = mlora.sgmv_workspace(T, 16, dev, n_proj=len(names))
 
     def fused():
-        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws, aligned=True)
+        plan = mlora.plan_prefill(*b["seg"], T, pool, workspace=b["ws"], aligned=True)
         mlora.gemm_lora([y[p] for p in names], [x_in[p] for p in names], [w[p] for p in names], pool, 0, names, plan)
 
     def unfused():
-        plan = mlora.plan_prefill(ss, sl, sa, T, pool, workspace=ws)
+        plan = mlora.plan_prefill(*b["seg"], T, pool, workspace=b["ws"])
         for p in names:
             torch.mm(x_in[p], w[p], out=y[p])
         mlora.sgmv_multi([y[p] for p in names], [x_in[p] for p in names], pool, 0, names, plan)
@@ -243,40 +398,90 @@ def bench_f1(args, dev):
         for p in names:
             torch.mm(x_in[p], w[p], out=y[p])
 
-    def timed(fn):
-        fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for _ in range(args.warmup):
-            fn()
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(args.steps):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / args.steps
-
-    ms_unfused = timed(unfused)
-    ms_base = timed(base_only)
-    ms_per_step = timed(fused)
+    reps = reps_for(fused, steps, min_ms) if min_ms else steps
+    side = max(5, min(reps, steps))
+    ms_unfused = timed(unfused, side, warmup)["ms"]
+    ms_base = timed(base_only, side, warmup)["ms"]
+    t = timed(fused, reps, warmup)
+    ms_per_step = t["ms"]
     flops = sum(2.0 * T * hin * hout + 2.0 * 64 * (hin + hout) * T for hin, hout in projections.values())
+    # every operand once: x, W, y written, the touched adapters' rows
+    hbm_bytes = sum(T * hin * 2 + hin * hout * 2 + T * hout * 2 for hin, hout in projections.values())
     tflops = flops / (ms_per_step * 1e-3) / 1e12
-    out = {"metric": "base projection + LoRA prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
-           "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-           "config": {"workload": "config-4 batch with base weights: Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
-                                  "32 rank-64 adapters, bf16; y = x W + delta in one pass", "tokens": T, "segments": 16,
-                      "library_gemm_then_sgmv_ms": ms_unfused, "library_gemm_alone_ms": ms_base,
-                      "speedup_over_library_gemm_then_sgmv": ms_unfused / ms_per_step},
-           "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                        "frac": tflops / MFMA_PEAK_BF16_TFLOPS, "traffic": None,
-                        "kernel": "sgmv shrink + scaled reduce + gemm_lora_kernel (one launch over the 7 projections)",
-                        "flops_per_step": flops},
-           "cpu_baseline": None if args.no_cpu else cpu_baseline_prefill(True)}
-    print(json.dumps(out), flush=True)
+    return {"metric": "base projection + LoRA prefill throughput", "value": tflops, "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": reps, "warmup": warmup, "ms_per_step": ms_per_step,
+            "ms_per_step_spread": {k: t[k] for k in ("p10", "p50", "p90")}, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "config-4 batch with base weights: Llama-13B q/k/v/o/gate/up/down, 16 requests U[128,1024], "
+                                   "32 rank-64 adapters, bf16; y = x W + delta in one pass", "tokens": T, "segments": 16,
+                       "form": "shrink + scaled reduce + one GEMM launch over the 7 projections",
+                       "library_gemm_then_sgmv_ms": ms_unfused, "library_gemm_alone_ms": ms_base,
+                       "speedup_over_library_gemm_then_sgmv": ms_unfused / ms_per_step},
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": MFMA_PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / MFMA_PEAK_BF16_TFLOPS, "traffic": None, "traffic_source": None,
+                         "kernel": "sgmv shrink + scaled reduce + gemm_lora_kernel (one launch over the 7 projections)",
+                         "flops_per_step": flops, "mfma_frac": tflops / MFMA_PEAK_BF16_TFLOPS,
+                         "hbm_frac": hbm_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, "operand_bytes_per_step": hbm_bytes},
+            "cpu_baseline": cpu_baseline_prefill(True) if cpu else None}
 
 
+# ---------------------------------------------------------------------------------------------- reference layout
+def bench_reflayout(args, dev, steps, warmup, min_ms=0.0):
+    """The reference's own decode call on its own pool layout (lora_gpu.py:33-40,122-163) at config-2 size: q, k, v
+    of one layer, pool tensors [N, L, r, Hin] / [N, L, Hout, r], int64 indices, y = zeros then y += delta
+    (`Lora_GPU.invoke_one_layer_{q,k,v}`), 32 layers per step, eager as the reference calls it and from a HIP graph."""
+    import numpy as np
+    import torch
+
+    import mlora
+    from mlora import workloads
+    T, N, L, r, H = 256, 64, 32, 16, 4096
+    rng = np.random.default_rng(1002)
+    cfg = dict(n_layers=L, batch_size=N, lora_rank=r, hidden_dim=H, tp_degree=1, max_prefill_batch_size=1)
+    gpu = mlora.Lora_GPU(cfg, device=dev, seed=7)
+    ids = torch.from_numpy(workloads.zipf_adapters(rng, T, N, 1.0).astype(np.int64)).to(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(2002)
+    xs = [torch.randn(T, H, device=dev, generator=gen).half() for _ in range(L)]
+
+    batched = getattr(gpu, "invoke_one_layer_qkv", None) if not args.fused else None    # --fused: one call per projection
+
+    def step():
+        for l in range(L):
+            if batched is not None:
+                batched(xs[l], l, lora_ids=ids)
+            else:
+                for f in (gpu.invoke_one_layer_q, gpu.invoke_one_layer_k, gpu.invoke_one_layer_v):
+                    f(xs[l], l, False, lora_ids=ids)
+
+    step()
+    torch.cuda.synchronize()
+    reps = reps_for(step, steps, min_ms) if min_ms else steps
+    eager = timed(step, reps, warmup)
+    # under a graph the output buffers are those of the capture
+    run = graph_of(step)
+    greps = reps_for(run, steps, min_ms) if min_ms else steps
+    t = timed(run, greps, warmup)
+    uniq = np.unique(ids.cpu().numpy())
+    # x is read once for q, k, v; y is written, not read (the call starts from zeros); indices are int64
+    alg = T * H * 2 + 3 * T * H * 2 + 3 * len(uniq) * r * (H + H) * 2 + 8 * T
+    launch_us = t["ms"] * 1e3 / L
+    achieved = alg / (launch_us * 1e-6) / 1e9
+    return {"metric": "BGMV decode throughput on the reference's pool layout", "value": T * 3 * L / (t["ms"] * 1e-3),
+            "unit": "token-projections/s", "n_gpus": 1, "steps": greps, "warmup": warmup, "ms_per_step": t["ms"],
+            "ms_per_step_spread": {k: t[k] for k in ("p10", "p50", "p90")}, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "reference layout, config-2 size: q/k/v 4096->4096, 256 tokens, 64 rank-16 adapters, Zipf(1.0), "
+                                   "fp16, pool [N,L,r,Hin] / [N,L,Hout,r], int64 indices", "layers": L, "tokens": T,
+                       "form": "one q/k/v call per layer" if batched is not None else "one call per projection", "hip_graph": True,
+                       "eager_ms_per_step": eager["ms"], "eager_spread": {k: eager[k] for k in ("p10", "p50", "p90")}},
+            "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                         "traffic": None, "traffic_source": None, "kernel": "one layer's q/k/v calls on the reference layout",
+                         "launch_us": launch_us, "algorithmic_bytes_per_launch": alg},
+            "cpu_baseline": None}
+
+
+# ---------------------------------------------------------------------------------------------- swap-in, transport
 def bench_swap(args, dev):
     """Adapter swap-in (cold start): one rank-64 adapter for q/k/v of a 32-layer, hidden-4096 model (the shape the
     reference's swapper is started with, shared_tensor.py:23-30) from pinned host memory onto its pool pages.
@@ -335,31 +540,32 @@ def bench_swap(args, dev):
     ref_t = sum(ref_style(i % 4) for i in range(n_ref)) / n_ref
 
     gbs = nbytes / total / 1e9
-    out = {"metric": "adapter swap-in throughput (host pinned -> pool pages)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
-           "steps": args.steps, "warmup": args.warmup, "ms_per_step": total * 1e3, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
-           "config": {"workload": "swap-in of one rank-64 adapter, q/k/v, 32 layers, hidden 4096, fp16",
-                      "bytes_per_adapter": nbytes, "layers_per_copy": loader.layers_per_copy,
-                      "ms_until_layers_8_15_ready": first * 1e3, "ms_host_time_to_issue": issue * 1e3},
-           "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
-                        "kernel": "host->device copies (copy engine) + scatter_kernel"},
-           "cpu_baseline": {"value": nbytes / ref_t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                            "sample": f"the swapper's copy pattern (pageable host tensors, one copy and one slice assignment per "
-                                      f"layer and tensor) restated with torch, {n_ref} adapters, {ref_t * 1e3:.2f} ms each"}}
-    print(json.dumps(out), flush=True)
+    return {"metric": "adapter swap-in throughput (host pinned -> pool pages)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": total * 1e3,
+            "ms_per_step_spread": percentiles([r_[2] * 1e3 for r_ in res]), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
+            "config": {"workload": "swap-in of one rank-64 adapter, q/k/v, 32 layers, hidden 4096, fp16",
+                       "bytes_per_adapter": nbytes, "layers_per_copy": loader.layers_per_copy,
+                       "ms_until_layers_8_15_ready": first * 1e3, "ms_host_time_to_issue": issue * 1e3},
+            "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
+                         "traffic_source": None, "kernel": "host->device copies (copy engine) + scatter_kernel"},
+            "cpu_baseline": {"value": nbytes / ref_t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                             "sample": f"the swapper's copy pattern (pageable host tensors, one copy and one slice assignment per "
+                                       f"layer and tensor) restated with torch, {n_ref} adapters, {ref_t * 1e3:.2f} ms each"}}
 
 
 def bench_assist(args, dev):
-    """CPU-assist transport alone (no worker arithmetic): hidden states of a prefill batch to the host request
-    slots plus the wake-up codes, and the q/k/v result slots back to the device.  Shape of the reference's
-    CPU-assisted prefill: hidden 4096, slots of 256 tokens, 64 tokens per worker; 8 requests of 256 tokens.
-    Beside it, the reference's call pattern restated with torch (one device->host copy per request, one
-    host->device copy per finished chunk and projection, lora_cpu.py:176-232)."""
+    """CPU-assisted prefill of the reference's shape (hidden 4096, slots of 256 tokens, 64 tokens per worker; 8 requests
+    of 256 tokens): hidden states to the host request slots plus the wake-up codes, the q/k/v chunks on the package's
+    in-process workers (libmlora_cpu.so), and the result slots back to the device.  The transport alone is timed with
+    the signals cleared by hand.  Beside it, the reference's call pattern restated with torch (one device->host copy
+    per request, one host->device copy per finished chunk and projection, lora_cpu.py:176-232)."""
+    import numpy as np
     import torch
 
     import mlora
-    B, tkn, H, cap = 8, 256, 4096, 64
-    cfg = dict(batch_size=B, lora_num=64, tp_degree=1, hidden_dim=H, lora_rank=16, token_per_lora=cap, n_layers=32)
+    B, tkn, H, cap, r = 8, 256, 4096, 64, 16
+    cfg = dict(batch_size=B, lora_num=64, tp_degree=1, hidden_dim=H, lora_rank=r, token_per_lora=cap, n_layers=32)
     cpu = mlora.Lora_CPU(cfg, gpu_id=0, device=dev)
     hidden = torch.randn(B * tkn, H, device=dev).half()
     e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
@@ -379,6 +585,23 @@ def bench_assist(args, dev):
             t_imp += e[2].elapsed_time(e[3])
     t_exp, t_imp = t_exp / args.steps, t_imp / args.steps
     b_exp, b_imp = B * tkn * H * 2, 3 * B * tkn * H * 2
+
+    # the whole CPU-assisted call with the in-process workers: export -> 3 x 32 chunks of 64 tokens on the host cores -> import
+    rng = np.random.default_rng(77)
+    down = [(rng.standard_normal((1, H, r)) * 0.001).astype(np.float32) for _ in range(3)]
+    up = [(rng.standard_normal((1, r, H)) * 0.001).astype(np.float32) for _ in range(3)]
+    n_threads = max(1, min(host_cores()["usable_by_this_process"], 64))
+    cpu.start_workers(down, up, n_threads=n_threads)
+    whole = []
+    for i in range(3 + max(3, args.steps // 4)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cpu.invoke_lora_async(hidden, tkn)
+        cpu.collect_qkv(tkn, B)
+        torch.cuda.synchronize()
+        if i >= 3:
+            whole.append((time.perf_counter() - t0) * 1e3)
+    cpu.stop_workers()
 
     # reference call pattern, restated: pinned host tensors, one copy per request out, one per chunk back
     slots = torch.empty((64, 256, H), dtype=torch.float16, pin_memory=True)
@@ -405,78 +628,23 @@ def bench_assist(args, dev):
     r_exp, r_imp = sum(x[0] for x in rr) / len(rr) * 1e3, sum(x[1] for x in rr) / len(rr) * 1e3
     cpu.close()
     gbs = (b_exp + b_imp) / ((t_exp + t_imp) * 1e-3) / 1e9
-    out = {"metric": "CPU-assist transport throughput (device <-> pinned host slots)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
-           "steps": args.steps, "warmup": args.warmup, "ms_per_step": t_exp + t_imp, "higher_is_better": True,
-           "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
-           "config": {"workload": "8 requests x 256 tokens, hidden 4096: export 16.8 MB + wake-up codes, import q/k/v 50.3 MB",
-                      "export_ms": t_exp, "import_ms": t_imp, "export_GBs": b_exp / t_exp / 1e6, "import_GBs": b_imp / t_imp / 1e6},
-           "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
-                        "kernel": "assist_export_kernel + assist_signal_kernel, assist_import_kernel"},
-           "cpu_baseline": {"value": (b_exp + b_imp) / ((r_exp + r_imp) * 1e-3) / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                            "sample": f"the reference's call pattern restated with torch: {B} copies out ({r_exp:.3f} ms), "
-                                      f"{3 * B * cpr} synchronous chunk copies back ({r_imp:.3f} ms)"}}
-    print(json.dumps(out), flush=True)
+    return {"metric": "CPU-assist transport throughput (device <-> pinned host slots)", "value": gbs, "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": t_exp + t_imp, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "u16", "data": "synthetic",
+            "config": {"workload": "8 requests x 256 tokens, hidden 4096: export 16.8 MB + wake-up codes, import q/k/v 50.3 MB",
+                       "export_ms": t_exp, "import_ms": t_imp, "export_GBs": b_exp / t_exp / 1e6, "import_GBs": b_imp / t_imp / 1e6,
+                       "whole_call_with_in_process_workers_ms": percentiles(whole), "worker_threads": n_threads},
+            "roofline": {"bound": "pcie", "achieved": gbs, "peak": 64.0, "unit": "GB/s", "frac": gbs / 64.0, "traffic": None,
+                         "traffic_source": None, "kernel": "assist_export_kernel + assist_signal_kernel, assist_import_kernel"},
+            "cpu_baseline": {"value": (b_exp + b_imp) / ((r_exp + r_imp) * 1e-3) / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                             "sample": f"the reference's call pattern restated with torch: {B} copies out ({r_exp:.3f} ms), "
+                                       f"{3 * B * cpr} synchronous chunk copies back ({r_imp:.3f} ms)"}}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
-    ap.add_argument("--group", type=int, default=-1,
-                    help="tokens of one adapter per work item (0 = no plan, one token each; default: by batch size)")
-    ap.add_argument("--split", action="store_true", help="decode: force the shrink + expand pair also where the host layer would pick the fused launch")
-    ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
-                         "instead of one call over the seven")
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--calib-copy", action="store_true",
-                    help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "swap", "assist", "f1"],
-                    help="c2 = decode BGMV (the headline metric); c1, c3 = the other decode configurations; "
-                         "c4 = prefill SGMV on Llama-13B shapes; c5 = full 32-layer step with 1000 adapters (about 165 GB); "
-                         "mafN = decode batch drawn from the reference's adapter-popularity vector of N adapters; "
-                         "swap = adapter swap-in from pinned host memory; assist = CPU-assist transport; "
-                         "f1 = base projection + LoRA in one pass on the config-4 batch, with the library GEMM + SGMV sequence timed beside it")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
-
-    import numpy as np
-    import torch
-
-    import mlora
-    from mlora import workloads
-
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
-    mlora._ext.lib()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if args.calib_copy:
-        src = torch.ones(128 << 20, dtype=torch.float16, device=dev)      # 256 MiB read + 256 MiB written per copy
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    if args.workload == "c4":
-        return bench_c4(args, dev)
-    if args.workload == "f1":
-        return bench_f1(args, dev)
-    if args.workload == "swap":
-        return bench_swap(args, dev)
-    if args.workload == "assist":
-        return bench_assist(args, dev)
-    return bench_decode(args, dev)
-
-
-# Decode workloads.  `inputs` names the activation tensor each projection reads (projections that
-# read the same tensor in the model share it here).  `layers` is chosen so that a step's working
-# set is far larger than the 256 MB last-level cache.
+# ---------------------------------------------------------------------------------------------- decode workloads
+# `inputs` names the activation tensor each projection reads (projections that read the same tensor in the
+# model share it here).  `layers` is chosen so that a step's working set is far larger than the 256 MB
+# last-level cache.
 _IN = {"q": "attn", "k": "attn", "v": "attn", "o": "o", "gate": "ffn", "up": "ffn", "down": "down"}
 DECODE = {
     "c1": dict(desc="config 1: single LoRA-delta op, q_proj 4096->4096, 32 decode tokens, 8 rank-16 adapters, "
@@ -506,27 +674,28 @@ for _n in (128, 256, 512):
         popularity=os.path.join(ROOT, "tests", "golden", f"maf_popularity_{_n}.npy"))
 
 
-def bench_decode(args, dev):
+def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
+    """One decode workload: its full JSON line.  With min_ms > 0 the step is repeated until the timed region is that
+    long (legs); otherwise exactly `steps` steps are timed."""
     import numpy as np
     import torch
 
     import mlora
     from mlora import workloads
 
-    cfg = DECODE[args.workload]
-    if args.group < 0:
-        args.group = mlora.ops.default_group(cfg["T"])
+    cfg = DECODE[workload]
+    group = args.group if args.group >= 0 else mlora.ops.default_group(cfg["T"])
     L = args.layers if args.layers > 0 else cfg["layers"]
     shapes = workloads.LLAMA7B_ATTN if cfg["shapes"] == "7b_attn" else workloads.LLAMA7B_ALL
     projs = cfg["projs"]
     shapes = {p: shapes[p] for p in projs}
     rng = np.random.default_rng(cfg["seed"])
     ranks = cfg["ranks"] if cfg["ranks"] is not None else rng.choice([8, 16, 32, 64], size=cfg["N"]).astype(np.int32)
-    log(f"building {args.workload} with {L} layers ...")
+    log(f"building {workload} with {L} layers ...")
     lora_ids = None
     if cfg.get("popularity"):
         lora_ids = workloads.draw_lora_ids(np.load(cfg["popularity"], allow_pickle=False), cfg["T"], seed=0)
-    wl = workloads.make_decode(args.workload, shapes, L, cfg["T"], cfg["N"], ranks, cfg["alpha"], seed=cfg["seed"],
+    wl = workloads.make_decode(workload, shapes, L, cfg["T"], cfg["N"], ranks, cfg["alpha"], seed=cfg["seed"],
                                device=dev, alpha_lora=32.0, tok_adapter=lora_ids)
     pool, T = wl.pool, len(wl.tok_adapter)
     log(f"pool slabs: {sum(t.numel() * 2 for t in list(pool.a_rows.values()) + list(pool.b_rows.values())) / 1e9:.2f} GB")
@@ -537,9 +706,9 @@ def bench_decode(args, dev):
     width = {_IN[p]: shapes[p][0] for p in projs}
     xs = [{i: torch.randn(T, width[i], device=dev, generator=gen).half() for i in inputs} for _ in range(L)]
     ys = [[torch.randn(T, shapes[p][1], device=dev, generator=gen).half() for p in projs] for _ in range(L)]
-    plan = mlora.plan_decode(tok, pool, group=args.group) if args.group else None
+    plan = mlora.plan_decode(tok, pool, group=group) if group else None
     fused = bool(args.fused or plan is None or
-                 (not args.split and mlora.ops.decode_fused(T, args.group, len(projs), pool.n_slots)))
+                 (not args.split and mlora.ops.decode_fused(T, group, len(projs), pool.n_slots)))
 
     # config 5 carries prefill segments through SGMV in the same step (activations shared by the layers:
     # they are larger than the last-level cache anyway)
@@ -562,7 +731,7 @@ def bench_decode(args, dev):
 
     def step():
         if plan is not None:
-            mlora.plan_decode(tok, pool, group=args.group, out=plan)
+            mlora.plan_decode(tok, pool, group=group, out=plan)
         if pre is None:
             bgmv_layers()
             return
@@ -573,33 +742,10 @@ def bench_decode(args, dev):
 
     step()
     torch.cuda.synchronize()
-
-    def make_runner(fn):
-        if args.no_graph:
-            return fn
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            fn()
-        return g.replay
-
-    def timed(run, reps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record()
-        for _ in range(reps):
-            run()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1)          # ms, on the stream the kernels run on
-
-    run_step = make_runner(step)
-    for _ in range(args.warmup):
-        run_step()
-    torch.cuda.synchronize()
-    t_wall = time.perf_counter()
-    ms = timed(run_step, args.steps)
-    wall = time.perf_counter() - t_wall
-    ms_per_step = ms / args.steps
+    run_step = graph_of(step, not args.no_graph)
+    reps = reps_for(run_step, steps, min_ms) if min_ms else steps
+    t = timed(run_step, reps, warmup)
+    ms_per_step = t["ms"]
     n_tok = T + (pre["T"] if pre else 0)
     value = n_tok * len(projs) * L / (ms_per_step * 1e-3)
 
@@ -608,47 +754,157 @@ def bench_decode(args, dev):
     alg = algorithmic_bytes(T, shp, wl.ranks[uniq])
     per_token_gather = sum(T * h[0] * 2 + 2 * T * h[1] * 2 + int(wl.ranks[wl.tok_adapter].sum()) * (h[0] + h[1]) * 2 + 4 * T
                            for h in shp)
-    if pre is None:
-        # The BGMV calls alone: the same layers without the gather, for the roofline figure.
-        run_bgmv = make_runner(bgmv_layers)
-        for _ in range(args.warmup):
-            run_bgmv()
-        ms_k = timed(run_bgmv, args.steps)
-        launch_us = ms_k * 1e3 / (args.steps * L)
-        achieved = alg / (launch_us * 1e-6) / 1e9
-        kernel = ("bgmv_kernel" if fused else "bgmv_shrink_kernel + bgmv_expand_kernel (one layer's pair)") + \
-                 f", {len(projs)} projections per call"
-        extra = {"launch_us": launch_us, "algorithmic_bytes_per_launch": alg,
-                 "per_token_gather_bytes_per_launch": per_token_gather}
-    else:
+    # The BGMV calls alone (the same layers without gather, plan and prefill launches): the roofline figure.
+    run_bgmv = graph_of(bgmv_layers, not args.no_graph)
+    tk = timed(run_bgmv, reps_for(run_bgmv, steps, min_ms) if min_ms else steps, warmup)
+    launch_us = tk["ms"] * 1e3 / L
+    achieved = alg / (launch_us * 1e-6) / 1e9
+    kernel = ("bgmv_kernel" if fused else "bgmv_shrink_kernel + bgmv_expand_kernel (one layer's pair)") + \
+             f", {len(projs)} projections per call"
+    extra = {"launch_us": launch_us, "launch_us_spread": {k: tk[k] * 1e3 / L for k in ("p10", "p50", "p90")},
+             "algorithmic_bytes_per_launch": alg, "per_token_gather_bytes_per_launch": per_token_gather}
+    if pre is not None:
         # Mixed step: decode and prefill bytes of all layers over the whole step (gather and plan included).
         pu = np.unique(pre["adapters"])
         alg_pre = algorithmic_bytes(pre["T"], shp, wl.ranks[pu]) + 12 * len(pre["adapters"]) * len(projs)
         alg_step = (alg + alg_pre) * L
-        achieved = alg_step / (ms_per_step * 1e-3) / 1e9
-        kernel = "whole step: gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"
-        extra = {"algorithmic_bytes_per_step": alg_step, "decode_bytes_per_layer": alg, "prefill_bytes_per_layer": alg_pre}
-    traffic = MEASURED_TRAFFIC_C2 if (args.workload == "c2" and args.group == 4 and L == 32 and not fused) else None
+        extra.update({"whole_step": {"achieved": alg_step / (ms_per_step * 1e-3) / 1e9,
+                                     "frac": alg_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                                     "algorithmic_bytes_per_step": alg_step, "prefill_bytes_per_layer": alg_pre,
+                                     "kernels": "gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"}})
+    traffic, src = traffic_of(workload, group == 4 and L == cfg["layers"] and not fused)
 
     out = {
         "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",
-        "value": value, "unit": "token-projections/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": value, "unit": "token-projections/s", "n_gpus": 1, "steps": reps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "ms_per_step_spread": {k: t[k] for k in ("p10", "p50", "p90")},
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": cfg["desc"], "layers": L, "projections_per_call": len(projs),
                    "launches_per_step": L * (1 if fused else 2) + (1 if plan else 0) + ((1 + 3 * L) if pre else 0),
                    "form": "fused" if fused else "shrink + expand",
                    "tokens": T, "prefill_tokens": pre["T"] if pre else 0, "adapters": cfg["N"],
-                   "adapters_touched": int(len(uniq)), "group": args.group,
-                   "hip_graph": not args.no_graph, "wall_s_timed_region": wall},
+                   "adapters_touched": int(len(uniq)), "group": group,
+                   "hip_graph": not args.no_graph, "timed_region_ms": t["timed_ms"], "wall_s_timed_region": t["wall_s"]},
         "roofline": dict({"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                          "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "kernel": kernel}, **extra),
+                          "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": src, "kernel": kernel}, **extra),
         "cpu_baseline": None,
     }
+    if args.eager and not args.no_graph:
+        te = timed(step, max(5, min(reps, 50)), 2)
+        out["config"]["eager_ms_per_step"] = te["ms"]
+    return out
+
+
+def leg_of(line):
+    """The part of a workload's line that goes into the headline's `legs` object."""
+    keep = {k: line[k] for k in ("metric", "value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "dtype")}
+    keep["workload"] = line["config"]["workload"]
+    keep["form"] = line["config"].get("form")
+    for k in ("eager_ms_per_step", "library_gemm_then_sgmv_ms", "speedup_over_library_gemm_then_sgmv", "tokens", "adapters_touched",
+              "steps_in_trace", "adapters_touched_per_step", "swap_ins"):
+        if k in line["config"]:
+            keep[k] = line["config"][k]
+    keep["roofline"] = line["roofline"]
+    return keep
+
+
+SINGLE = ["c1", "c2", "c3", "c4", "c5", "maf128", "maf256", "maf512", "maf_trace", "swap", "assist", "f1", "reflayout"]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=0, help="layers per step (0 = the workload's own count)")
+    ap.add_argument("--group", type=int, default=-1,
+                    help="tokens of one adapter per work item (0 = no plan, one token each; default: by batch size)")
+    ap.add_argument("--split", action="store_true", help="decode: force the shrink + expand pair also where the host layer would pick the fused launch")
+    ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
+                         "instead of one call over the seven")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--eager", action="store_true", help="decode: also time the step launched eagerly (config.eager_ms_per_step)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-legs", action="store_true", help="default run: the config-5 headline alone")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (known size) so that a counter run can be scaled")
+    ap.add_argument("--workload", default="all", choices=["all"] + SINGLE,
+                    help="all (default) = config 5 as the headline plus the legs c1, c2, c3, c4, f1, reflayout, maf_trace; a name = that "
+                         "workload alone: c1..c3, c5 decode BGMV; c4 prefill SGMV on Llama-13B shapes; mafN = decode batch drawn from the "
+                         "reference's adapter-popularity vector of N adapters; maf_trace = continuous-batching decode sequence from the "
+                         "reference's arrival trace; swap = adapter swap-in from pinned host memory; assist = CPU-assist transport; "
+                         "f1 = base projection + LoRA in one pass on the config-4 batch; reflayout = the reference's pool layout and call")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import mlora
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    mlora._ext.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.calib_copy:
+        src = torch.ones(128 << 20, dtype=torch.float16, device=dev)      # 256 MiB read + 256 MiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    def one(workload, steps, warmup, min_ms, cpu):
+        if workload == "c4":
+            return bench_c4(args, dev, steps, warmup, min_ms, cpu)
+        if workload == "f1":
+            return bench_f1(args, dev, steps, warmup, min_ms, cpu)
+        if workload == "reflayout":
+            return bench_reflayout(args, dev, steps, warmup, min_ms)
+        if workload == "maf_trace":
+            from mlora import trace_driver
+            return trace_driver.bench_trace(args, dev, steps, warmup)
+        if workload == "swap":
+            return bench_swap(args, dev)
+        if workload == "assist":
+            return bench_assist(args, dev)
+        line = bench_decode(args, dev, workload, steps, warmup, min_ms)
+        if cpu:
+            log("timing the CPU baseline ...")
+            line["cpu_baseline"] = cpu_baseline()
+        return line
+
+    if args.workload != "all":
+        print(json.dumps(one(args.workload, args.steps, args.warmup, 0.0, not args.no_cpu)), flush=True)
+        return
+
+    t_start = time.perf_counter()
+    legs = {}
+    ceiling = stream_ceiling(dev)
+    if not args.no_legs:
+        args.eager = True
+        for w in ("c1", "c2", "c3", "c4", "f1", "reflayout", "maf_trace"):
+            log(f"leg {w} ...")
+            try:
+                legs[w] = leg_of(one(w, args.steps, args.warmup, MIN_LEG_MS, False))
+            except ImportError as exc:                    # a leg whose driver is not in this tree is reported, not hidden
+                legs[w] = {"error": str(exc)}
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+        args.eager = False
+    log("headline: config 5 ...")
+    line = bench_decode(args, dev, "c5", args.steps, args.warmup, 0.0)
+    line["stream_ceiling"] = ceiling
+    line["legs"] = legs
     if not args.no_cpu:
         log("timing the CPU baseline ...")
-        out["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(out), flush=True)
+        line["cpu_baseline"] = cpu_baseline()
+    line["config"]["bench_wall_s"] = time.perf_counter() - t_start
+    print(json.dumps(line), flush=True)
 
 
 if __name__ == "__main__":

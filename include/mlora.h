@@ -122,6 +122,14 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
                        int elt_bytes, void *stream);
 
 /*
+ * Measurement helper, no counterpart in the reference: one plain streaming pass over `bytes` of device memory
+ * (mode 0: read every 16 bytes once with nontemporal loads; mode 1: read, change and write back in place), so
+ * that a benchmark can print what a memory-bound launch reaches on the device at hand beside the LoRA kernels'
+ * figures.  Mode 1 adds 1 to the first 32-bit word of every 16 bytes.
+ */
+int mlora_probe_stream(void *buf, int64_t bytes, int mode, void *stream);
+
+/*
  * CPU-assist transport: the GPU side of the path on which host workers compute the LoRA delta while an
  * adapter is still loading (HIP equivalents of the reference's tensor_cp copy family,
  * csrc/cuda_ops.hpp:109-229; no arithmetic here -- the workers are the reference's own processes or any

@@ -70,6 +70,40 @@ def test_assist_round_trip(batch, tkn, cap, tp, gpu_id):
         cpu.close()
 
 
+@pytest.mark.parametrize("batch,tkn,cap,tp,gpu_id,threads", [(3, 20, 8, 2, 1, 4), (8, 64, 16, 1, 0, 8), (2, 256, 64, 4, 2, 3)])
+def test_assist_end_to_end_with_the_in_process_workers(batch, tkn, cap, tp, gpu_id, threads):
+    """Export -> the package's own host workers (libmlora_cpu.so thread pool) -> import, two batches in a row
+    through the same slots, each against the oracle's worker arithmetic, bit for bit."""
+    rng = np.random.default_rng(900 + batch * tkn)
+    H, r, N = 512, 16, 5
+    cfg = dict(batch_size=batch, lora_num=32, tp_degree=tp, hidden_dim=H, lora_rank=r, token_per_lora=cap, n_layers=2)
+    cpu = Lora_CPU(cfg, gpu_id=gpu_id)
+    try:
+        down = [(rng.standard_normal((N, H, r)) * 0.05).astype(np.float32) for _ in range(3)]
+        up = [(rng.standard_normal((N, r, H)) * 0.05).astype(np.float32) for _ in range(3)]
+        slot_adapter = rng.integers(0, N, cpu.lora_num).astype(np.int32)
+        cpu.start_workers(down, up, n_threads=threads, slot_adapter=slot_adapter)
+        out = H // tp
+        n_chunks = 0
+        for rep, (b, t) in enumerate(((batch, tkn), (max(1, batch - 1), max(1, tkn // 2)))):
+            hidden = torch.randn(b * t, H, device="cuda", dtype=torch.float16)
+            h_bits = hidden.cpu().numpy().view(np.uint16).reshape(b, t, H)
+            say(f"assist end to end: batch={b} tkn={t} cap={cap} threads={threads} (call {rep})")
+            cpu.invoke_lora_async(hidden, t, layer_id=rep)
+            res = cpu.collect_qkv(t, b, timeout_s=30.0)
+            torch.cuda.synchronize()
+            n_chunks += 3 * b * ((t - 1) // cap + 1)
+            for p, got in enumerate(res):
+                assert got.shape == (b, t, out)
+                for i in range(b):
+                    a = slot_adapter[i]
+                    want = orc.cpu_lora_worker(np.ascontiguousarray(h_bits[i]), down[p][a], up[p][a])[:, out * gpu_id:out * (gpu_id + 1)]
+                    assert np.array_equal(got[i].cpu().numpy().view(np.uint16), want), (rep, p, i)
+        assert cpu.stop_workers() == (n_chunks, 0)
+    finally:
+        cpu.close()
+
+
 def test_assist_rejects_what_does_not_fit():
     cfg = dict(batch_size=4, lora_num=4, tp_degree=1, hidden_dim=64, lora_rank=8, token_per_lora=8, n_layers=1)
     cpu = Lora_CPU(cfg)
