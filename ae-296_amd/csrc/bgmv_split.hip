@@ -23,6 +23,15 @@
 namespace mlora {
 
 
+// How a launch treats the adapter rows, chosen by the host from the size of the batch:
+//   BIG = false: a hot adapter's work items all run at once (the launch is about one round of workgroups), rows
+//     pass through L2 once and are read with the nontemporal hint so that they do not displace records and sums;
+//   BIG = true: the launch is many rounds of workgroups, the items of a hot adapter follow each other on one XCD
+//     and find its rows in L2 only if they are kept: ordinary loads, and the expand keeps fewer rows in flight per
+//     lane (more resident wavefronts instead), which measured faster at that size.
+template <bool BIG>
+__device__ __forceinline__ uint4 ld_rows(const void *p) { if constexpr (BIG) return ldg16(p); else return ldg16_stream(p); }
+
 struct ItemId { int b, q; };
 
 __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
@@ -51,7 +60,7 @@ __device__ __forceinline__ int slice_factor(int r)
 // Shrink of one (item, projection, column slice) over the first 4 * NR rank rows (NR per 16-lane
 // row).  The caller picks the smallest NR that covers the item's rank, so an adapter of rank 8 in a
 // pool that goes up to rank 64 issues loads for 8 rows, not 64.
-template <int DT, int G, int RMAX, int KSC, int NR>
+template <int DT, int G, int RMAX, int KSC, int NR, bool BIG>
 __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__restrict__ rows, const int (&tok)[G],
                                             int r, int proj, int ks, int slot, float (&s_part)[4][G][RMAX])
 {
@@ -69,8 +78,13 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
     const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows[proj]);
 
     // Loads are unconditional: an absent rank row reads row 0 of the slab and a token slot beyond
-    // ntok reads token 0 (both discarded below); a chunk past the end of the row re-reads the
-    // last chunk with x forced to zero.
+    // ntok reads token 0 (both discarded below).  Each wavefront covers a quarter of the slice in steps
+    // of 16 chunks per 16-lane row.  A slice that lies inside the row (all but a projection's last one)
+    // is read at fixed distances from one address per row, so the loads need no address registers of
+    // their own; the last, partial slice re-reads the row's last chunk for chunks past the end, with x
+    // forced to zero.
+    const int c_first = kc0 + wave * (STEPS * 16) + cl;
+    const bool whole = kc0 + KSC <= ncc_in;                     // uniform over the workgroup
     const uint4 *ap[NR];
     unsigned row_ok = 0;
 #pragma unroll
@@ -78,44 +92,58 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
         int row = rows[rg + 4 * i];
         row = (row >= 0 && row < pv.n_rows_a) ? row : -1;
         row_ok |= (row >= 0 ? 1u : 0u) << i;
-        ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+        ap[i] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin) + (whole ? c_first : 0);
     }
     const uint4 *xp[G];
 #pragma unroll
-    for (int k = 0; k < G; k++) xp[k] = reinterpret_cast<const uint4 *>(x + (size_t)(tok[k] >= 0 ? tok[k] : 0) * hin);
+    for (int k = 0; k < G; k++)
+        xp[k] = reinterpret_cast<const uint4 *>(x + (size_t)(tok[k] >= 0 ? tok[k] : 0) * hin) + (whole ? c_first : 0);
     float acc[G][NR];
 #pragma unroll
     for (int k = 0; k < G; k++)
 #pragma unroll
         for (int i = 0; i < NR; i++) acc[k][i] = 0.f;
 
-    // Each wavefront covers a quarter of the slice in steps of 16 chunks per 16-lane row.
+    if (whole) {
 #pragma unroll
-    for (int it0 = 0; it0 < STEPS; it0 += U) {
-        uint4 xv[G][U];
-        uint4 av[NR][U];
-        bool cv[U];
+        for (int it0 = 0; it0 < STEPS; it0 += U) {
+            uint4 xv[G][U];
+            uint4 av[NR][U];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int c = kc0 + wave * (STEPS * 16) + (it0 + u) * 16 + cl;
-            cv[u] = c < ncc_in;
-            const int cs = c < ncc_in ? c : ncc_in - 1;
+            for (int u = 0; u < U; u++) {
 #pragma unroll
-            for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + cs);
+                for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + (it0 + u) * 16);
 #pragma unroll
-            for (int i = 0; i < NR; i++) av[i][u] = ldg16_stream(ap[i] + cs);
+                for (int i = 0; i < NR; i++) av[i][u] = ld_rows<BIG>(ap[i] + (it0 + u) * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int i = 0; i < NR; i++)
+#pragma unroll
+                    for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
         }
+    } else {
+#pragma unroll 1
+        for (int it = 0; it < STEPS; it++) {
+            const int c = c_first + it * 16;
+            const bool cv = c < ncc_in;
+            const int cs = cv ? c : ncc_in - 1;
+            uint4 xv[G];
+            uint4 av[NR];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
+            for (int k = 0; k < G; k++) xv[k] = ldg16_stream(xp[k] + cs);
+#pragma unroll
+            for (int i = 0; i < NR; i++) av[i] = ld_rows<BIG>(ap[i] + cs);
 #pragma unroll
             for (int k = 0; k < G; k++) {
-                xv[k][u].x = cv[u] ? xv[k][u].x : 0u; xv[k][u].y = cv[u] ? xv[k][u].y : 0u;
-                xv[k][u].z = cv[u] ? xv[k][u].z : 0u; xv[k][u].w = cv[u] ? xv[k][u].w : 0u;
+                xv[k].x = cv ? xv[k].x : 0u; xv[k].y = cv ? xv[k].y : 0u;
+                xv[k].z = cv ? xv[k].z : 0u; xv[k].w = cv ? xv[k].w : 0u;
             }
 #pragma unroll
             for (int i = 0; i < NR; i++)
 #pragma unroll
-                for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i][u], xv[k][u], acc[k][i]);
+                for (int k = 0; k < G; k++) acc[k][i] = dot8<DT>(av[i], xv[k], acc[k][i]);
         }
     }
 
@@ -139,20 +167,22 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
     }
 }
 
-template <int DT, int G, int RMAX, int KSC>
+template <int DT, int G, int RMAX, int KSC, bool BIG>
 __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
 {
     __shared__ float s_part[4][G][RMAX];
 
-    const ItemId id = split_id(blockIdx.x, p.n_proj * p.ks_max);
-    const int proj = id.q / p.ks_max, ks = id.q - proj * p.ks_max;
+    // workgroup -> (record, projection, slice): only the slices a projection has are numbered
+    const ItemId id = split_id(blockIdx.x, p.sh_end[p.n_proj - 1]);
+    int proj = 0;
+    while (proj + 1 < p.n_proj && id.q >= p.sh_end[proj]) proj++;
+    const int ks = id.q - (proj ? p.sh_end[proj - 1] : 0);
     const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
     int ntok = rec[0];
     if (ntok <= 0) return;
     ntok = ntok < G ? ntok : G;
     const int adapter = rec[1];
     if (adapter < 0) return;
-    if (ks * KSC >= (p.hin[proj] >> 3)) return;                 // this projection has fewer slices
     int r = rec[2];
     r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
     int tok[G];
@@ -169,7 +199,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     auto go = [&](auto nr_tag, auto f_tag) {
         constexpr int NR = decltype(nr_tag)::value, F = decltype(f_tag)::value;
         if (ks % F) return;
-        shrink_rows<DT, G, RMAX, KSC * F, NR>(p, rows, tok, r, proj, ks / F, ks, s_part);
+        shrink_rows<DT, G, RMAX, KSC * F, NR, BIG>(p, rows, tok, r, proj, ks / F, ks, s_part);
     };
     using SF = SliceFactor<RMAX>;
     if constexpr (RMAX >= 64) {
@@ -182,25 +212,27 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     go(std::integral_constant<int, 2>{}, std::integral_constant<int, SF::F2>{});
 }
 
-template <int DT, int G, int RMAX, int KSC, int NTE>
+template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 {
     constexpr int NT = NTE;                                    // one 16-byte chunk of the slice per thread
-    constexpr int EB = RMAX < 16 ? RMAX : 16;                   // B rank rows in flight per lane
+    constexpr int EBW = BIG ? 4 : 8;
+    constexpr int EB = RMAX < EBW ? RMAX : EBW;                 // B rank rows in flight per lane
     __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
 
     const int tid = threadIdx.x;
     const PoolView &pv = p.pool;
 
-    const ItemId id = split_id(blockIdx.x, p.n_proj * p.cs_max);
-    const int proj = id.q / p.cs_max, cs = id.q - proj * p.cs_max;
+    const ItemId id = split_id(blockIdx.x, p.ex_end[p.n_proj - 1]);
+    int proj = 0;
+    while (proj + 1 < p.n_proj && id.q >= p.ex_end[proj]) proj++;
+    const int cs = id.q - (proj ? p.ex_end[proj - 1] : 0);
     const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
     int ntok = rec[0];
     if (ntok <= 0) return;
     ntok = ntok < G ? ntok : G;
     const int hout = p.hout[proj];
     const int ncc_out = hout >> 3;
-    if (cs * NTE >= ncc_out) return;                   // this projection has fewer slices
     const int cc = cs * NTE + tid;
     const bool active = cc < ncc_out;
     const int adapter = rec[1];
@@ -242,15 +274,31 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         for (int jj = 0; jj < EB; jj++) out[jj] = (out[jj] >= 0 && out[jj] < pv.n_rows_b) ? out[jj] : -1;
     };
 
+    // A rank row's address is the same for the whole workgroup (scalar registers) and a lane adds its column
+    // offset; an absent row reads row 0 and is zeroed afterwards, so a batch of loads is issued without a branch.
+    const unsigned voff = (unsigned)(active ? cc : 0) * 16u;
+    auto load_b = [&](int j0, uint4 (&out)[EB]) {
+        int br[EB];
+        b_rows_of(j0, br);
+        if constexpr (!BIG) {
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++)
+                out[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+            return;
+        }
+#pragma unroll
+        for (int jj = 0; jj < EB; jj++) {
+            const int row = __builtin_amdgcn_readfirstlane(br[jj]);
+            const char *rp = reinterpret_cast<const char *>(brows) + (size_t)(row >= 0 ? row : 0) * (size_t)hout * 2u;
+            out[jj] = ldg16(rp + voff);
+            if (row < 0) out[jj] = zero16();
+        }
+    };
     // Everything the first step needs is requested before the partial sums are fetched.
     uint4 bv[EB];
     uint4 yv[G];
     if (active) {
-        int br[EB];
-        b_rows_of(0, br);
-#pragma unroll
-        for (int jj = 0; jj < EB; jj++)
-            bv[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+        load_b(0, bv);
 #pragma unroll
         for (int k = 0; k < G; k++)
             yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
@@ -263,8 +311,19 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         const int k = e / RMAX, j = e - k * RMAX;
         float s = 0.f;
         if (j < r && tok[k] >= 0) {
+            // eight slices' sums are requested at once (one round trip instead of one per slice) and added in
+            // ascending slice order
             const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
-            for (int ks = 0; ks < n_ks; ks += kstep) s += src[(size_t)ks * RMAX];
+            for (int ks0 = 0; ks0 < n_ks; ks0 += 8 * kstep) {
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    const int ks = ks0 + u * kstep;
+                    t[u] = ks < n_ks ? src[(size_t)ks * RMAX] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += t[u];
+            }
         }
         s_v[k][j] = s * scale;
     }
@@ -276,13 +335,7 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
     for (int k = 0; k < G; k++) unpack8<DT>(yv[k], o[k]);
 #pragma unroll 1
     for (int j0 = 0; j0 < r; j0 += EB) {
-        if (j0 > 0) {
-            int br[EB];
-            b_rows_of(j0, br);
-#pragma unroll
-            for (int jj = 0; jj < EB; jj++)
-                bv[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
-        }
+        if (j0 > 0) load_b(j0, bv);
 #pragma unroll
         for (int jj = 0; jj < EB; jj++) {
             float f[8];
@@ -300,17 +353,17 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
 }
 
-template <int DT, int G, int RMAX, int KSC, int NTE>
+template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 static int launch_pair(const BgmvArgs &a, hipStream_t s)
 {
-    const long long n_sh = (long long)a.n_proj * a.ks_max * a.items_cap;
-    const long long n_ex = (long long)a.n_proj * a.cs_max * a.items_cap;
+    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.items_cap;
+    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.items_cap;
     if (n_sh <= 0 || n_ex <= 0) return 0;
     if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC, BIG>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
     int rc = (int)hipGetLastError();
     if (rc) return rc;
-    hipLaunchKernelGGL((bgmv_expand_kernel<DT, G, RMAX, KSC, NTE>), dim3((unsigned)n_ex), dim3(NTE), 0, s, a);
+    hipLaunchKernelGGL((bgmv_expand_kernel<DT, G, RMAX, KSC, NTE, BIG>), dim3((unsigned)n_ex), dim3(NTE), 0, s, a);
     return (int)hipGetLastError();
 }
 
@@ -324,7 +377,11 @@ template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
 template <int DT, int G, int RMAX>
 static int launch_sliced(const BgmvArgs &a, hipStream_t s)
 {
-    return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE>(a, s);
+    // Rounds of shrink workgroups the launch may need (host's upper bound on the work items, three workgroups per
+    // compute unit): from about sixteen on, the items of a much-used adapter no longer run side by side.
+    const long long rounds = (long long)a.sh_end[a.n_proj - 1] * a.items_cap / (3 * 256);
+    if (rounds >= 16) return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, true>(a, s);
+    return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, false>(a, s);
 }
 void bgmv_split_slices(int max_rank, int *ksc, int *nte)
 {

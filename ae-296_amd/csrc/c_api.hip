@@ -343,6 +343,12 @@ static int bgmv_multi_impl(int n_proj, void *const *y, const void *const *x, con
         mlora::bgmv_split_slices(max_rank, &ksc, &nte);
         a.ks_max = (max_hin + ksc * 8 - 1) / (ksc * 8);
         a.cs_max = (max_hout + nte * 8 - 1) / (nte * 8);
+        int sh = 0, ex = 0;
+        for (int p = 0; p < n_proj; p++) {
+            sh += (hin[p] + ksc * 8 - 1) / (ksc * 8);
+            ex += (hout[p] + nte * 8 - 1) / (nte * 8);
+            a.sh_end[p] = sh; a.ex_end[p] = ex;
+        }
         rc = mlora::launch_bgmv_split(a, dtype, group, max_rank, static_cast<hipStream_t>(stream));
     } else {
         rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));

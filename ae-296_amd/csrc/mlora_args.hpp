@@ -51,8 +51,12 @@ struct BgmvArgs {
     int n_proj;
     int accumulate;
     float *vws;                    // two-launch form: partial sums [n_proj, T, ks_max, rank stride] (else nullptr)
-    int ks_max;                    // shrink slices of the widest hin
+    int ks_max;                    // shrink slices of the widest hin (stride of the partial sums)
     int cs_max;                    // expand slices of the widest hout
+    // two-launch form: the (projection, slice) pairs that exist, numbered consecutively; sh_end[p] / ex_end[p] is
+    // the number of shrink / expand slices of projections 0..p
+    int sh_end[MAX_PROJ];
+    int ex_end[MAX_PROJ];
 };
 
 constexpr int SCATTER_MAX_JOBS = 16;
