@@ -353,6 +353,191 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
 }
 
+// Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
+// with rank x slice width, so wider ranks take narrower slices (measured over 64 / 128 / 256 chunks
+// on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
+template <int RMAX> struct Slices;
+template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
+template <> struct Slices<32> { static constexpr int KSC = 128, NTE = 256; };
+template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
+// Sum over each aligned group of LPC lanes (1, 2, 4 or 8); every lane of the group gets the sum.
+template <int LPC>
+__device__ __forceinline__ float group_sum(float v)
+{
+    if constexpr (LPC >= 2) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));   // quad_perm [1,0,3,2]
+    if constexpr (LPC >= 4) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));   // quad_perm [2,3,0,1]
+    if constexpr (LPC >= 8) v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));  // row_half_mirror
+    return v;
+}
+
+// Expand on the reference's layout: B is given as one [hout, R] block per adapter and layer (wb_T_all of
+// lightllm/models/lora_gpu.py:34,37,40), i.e. the R values of an output column lie next to each other and the
+// columns of a slice form one contiguous run.  A workgroup walks its 2048-column slice in sub-tiles of 256
+// columns: the sub-tile's run of 256 * R values is read with fully coalesced 16-byte loads (chunk q = 256 i + t
+// holds 8 ranks of column q / (R / 8)), every lane multiplies its 8 ranks with the matching 8 intermediates of
+// each token, the R / 8 lanes of a column are added with DPP moves, and the sums pass through LDS so that y is
+// updated with 16-byte, row-contiguous accesses.  The next sub-tile's loads are in flight during the arithmetic.
+template <int DT, int G, int R, int KSC>
+__global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
+{
+    constexpr int RMAX = R <= 16 ? 16 : (R <= 32 ? 32 : 64);   // rank stride of the shrink's partial sums
+    constexpr int LPC = R / 8;                                  // lanes per column
+    constexpr int CPP = 256 / LPC;                              // columns per pass of 256 chunks
+    constexpr int SUB = 256;                                    // columns per sub-tile
+    constexpr int SLICE = 2048;                                 // columns per workgroup
+    __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
+    __shared__ __attribute__((aligned(16))) float s_out[2][G][SUB];
+
+    const int tid = threadIdx.x;
+    const ItemId id = split_id(blockIdx.x, p.ex_end[p.n_proj - 1]);
+    int proj = 0;
+    while (proj + 1 < p.n_proj && id.q >= p.ex_end[proj]) proj++;
+    const int cs = id.q - (proj ? p.ex_end[proj - 1] : 0);
+    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
+    int ntok = rec[0];
+    if (ntok <= 0) return;
+    ntok = ntok < G ? ntok : G;
+    const int hout = p.hout[proj];
+    const int adapter = rec[1];
+    int tok[G];
+#pragma unroll
+    for (int k = 0; k < G; k++) {
+        const int t = k < ntok ? rec[4 + k] : -1;
+        tok[k] = (t >= 0 && t < p.T) ? t : -1;
+    }
+    uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y[proj]);
+    const int col_begin = cs * SLICE;
+    const int col_end = col_begin + SLICE < hout ? col_begin + SLICE : hout;
+    // y rows are handled by the first G * 32 threads: thread t -> token t / 32, 8 columns from (t % 32) * 8 of the sub-tile
+    const int yk = tid >> 5, yc = (tid & 31) * 8;
+    int ytok = -1;
+#pragma unroll
+    for (int k = 0; k < G; k++) ytok = yk == k ? tok[k] : ytok;
+
+    if (adapter < 0 || adapter >= p.pool.n_adapters) {
+        if (!p.accumulate && ytok >= 0)
+            for (int c0 = col_begin; c0 < col_end; c0 += SUB)
+                if (c0 + yc < col_end) stg16(y + (size_t)ytok * hout + c0 + yc, zero16());
+        return;
+    }
+    const float scale = __builtin_bit_cast(float, rec[3]) * p.pool.uniform_scale;
+    const uint16_t *__restrict__ bt = static_cast<const uint16_t *>(p.b_rows[proj]) +
+                                      (size_t)adapter * (size_t)p.ref_layers * (size_t)hout * R;
+    const int part = tid % LPC;                                 // which 8 ranks of a column this lane multiplies
+
+    uint4 bv[LPC], bn[LPC];
+    auto load_sub = [&](int c0, uint4 (&out)[LPC]) {
+        // chunk 256 i + t of the sub-tile's run: column c0 + i * CPP + t / LPC, ranks part * 8 ..
+#pragma unroll
+        for (int i = 0; i < LPC; i++) {
+            const int col = c0 + i * CPP + tid / LPC;
+            out[i] = col < col_end ? ldg16_stream(bt + (size_t)c0 * R + ((size_t)i * 256 + tid) * 8) : zero16();
+        }
+    };
+    load_sub(col_begin, bv);
+    uint4 yv = zero16();
+    if (p.accumulate && ytok >= 0 && col_begin + yc < col_end) yv = ldg16_stream(y + (size_t)ytok * hout + col_begin + yc);
+
+    // v = scaling * (sum of the slices' partial sums), slices added in ascending order
+    const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
+    for (int e = tid; e < G * RMAX; e += 256) {
+        const int k = e / RMAX, j = e - k * RMAX;
+        float s = 0.f;
+        if (j < R && tok[k] >= 0) {
+            const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
+            for (int ks0 = 0; ks0 < n_ks; ks0 += 8) {
+                float t8[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) t8[u] = ks0 + u < n_ks ? src[(size_t)(ks0 + u) * RMAX] : 0.f;
+#pragma unroll
+                for (int u = 0; u < 8; u++) s += t8[u];
+            }
+        }
+        s_v[k][j] = s * scale;
+    }
+    __syncthreads();
+    float vr[G][8];                                             // this lane's 8 intermediates of every token
+#pragma unroll
+    for (int k = 0; k < G; k++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) vr[k][e] = s_v[k][part * 8 + e];
+
+    int buf = 0;
+#pragma unroll 1
+    for (int c0 = col_begin; c0 < col_end; c0 += SUB, buf ^= 1) {
+        const bool more = c0 + SUB < col_end;
+        if (more) load_sub(c0 + SUB, bn);
+        uint4 yn = zero16();
+        if (more && p.accumulate && ytok >= 0 && c0 + SUB + yc < col_end) yn = ldg16_stream(y + (size_t)ytok * hout + c0 + SUB + yc);
+#pragma unroll
+        for (int i = 0; i < LPC; i++) {
+            float f[8];
+            unpack8<DT>(bv[i], f);
+#pragma unroll
+            for (int k = 0; k < G; k++) {
+                float d = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) d = fmaf(vr[k][e], f[e], d);
+                d = group_sum<LPC>(d);
+                if (part == 0) s_out[buf][k][i * CPP + tid / LPC] = d;
+            }
+        }
+        __syncthreads();                                        // also orders this buffer's reads of two steps ago before these writes
+        if (ytok >= 0 && c0 + yc < col_end) {
+            float o[8];
+            unpack8<DT>(yv, o);                                 // zeros when not accumulating
+            const float4_t d0 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc]);
+            const float4_t d1 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc + 4]);
+            o[0] += d0[0]; o[1] += d0[1]; o[2] += d0[2]; o[3] += d0[3];
+            o[4] += d1[0]; o[5] += d1[1]; o[6] += d1[2]; o[7] += d1[3];
+            stg16_stream(y + (size_t)ytok * hout + c0 + yc, pack8<DT>(o));
+        }
+#pragma unroll
+        for (int i = 0; i < LPC; i++) bv[i] = bn[i];
+        yv = yn;
+    }
+}
+
+template <int DT, int G, int R>
+static int launch_pair_bt(const BgmvArgs &a, hipStream_t s)
+{
+    constexpr int RMAX = R <= 16 ? 16 : (R <= 32 ? 32 : 64);
+    constexpr int KSC = Slices<RMAX>::KSC;
+    static_assert(Slices<RMAX>::NTE * 8 == 2048, "the transposed-B expand walks 2048-column slices");
+    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.items_cap;
+    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.items_cap;
+    if (n_sh <= 0 || n_ex <= 0) return 0;
+    if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC, false>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL((bgmv_expand_bt_kernel<DT, G, R, KSC>), dim3((unsigned)n_ex), dim3(256), 0, s, a);
+    return (int)hipGetLastError();
+}
+
+template <int DT, int G>
+static int launch_bt_rank(const BgmvArgs &a, int r, hipStream_t s)
+{
+    switch (r) {
+    case 8: return launch_pair_bt<DT, G, 8>(a, s);
+    case 16: return launch_pair_bt<DT, G, 16>(a, s);
+    case 32: return launch_pair_bt<DT, G, 32>(a, s);
+    case 64: return launch_pair_bt<DT, G, 64>(a, s);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
+template <int DT>
+static int launch_bt_dt(const BgmvArgs &a, int group, int r, hipStream_t s)
+{
+    switch (group) {
+    case 1: return launch_bt_rank<DT, 1>(a, r, s);
+    case 2: return launch_bt_rank<DT, 2>(a, r, s);
+    case 4: return launch_bt_rank<DT, 4>(a, r, s);
+    default: return (int)hipErrorInvalidValue;
+    }
+}
+
 template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 static int launch_pair(const BgmvArgs &a, hipStream_t s)
 {
@@ -367,13 +552,6 @@ static int launch_pair(const BgmvArgs &a, hipStream_t s)
     return (int)hipGetLastError();
 }
 
-// Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
-// with rank x slice width, so wider ranks take narrower slices (measured over 64 / 128 / 256 chunks
-// on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
-template <int RMAX> struct Slices;
-template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
-template <> struct Slices<32> { static constexpr int KSC = 128, NTE = 256; };
-template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
 template <int DT, int G, int RMAX>
 static int launch_sliced(const BgmvArgs &a, hipStream_t s)
 {
@@ -416,6 +594,10 @@ int bgmv_split_rank_stride(int max_rank) { return max_rank <= 16 ? 16 : (max_ran
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s)
 {
     if (!a.work || !a.vws) return (int)hipErrorInvalidValue;
+    if (a.b_transposed) {
+        if (dtype == DT_F16) return launch_bt_dt<DT_F16>(a, group, max_rank, s);
+        return launch_bt_dt<DT_BF16>(a, group, max_rank, s);
+    }
     if (dtype == DT_F16) return launch_split_dt<DT_F16>(a, group, max_rank, s);
     return launch_split_dt<DT_BF16>(a, group, max_rank, s);
 }

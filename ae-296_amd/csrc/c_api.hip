@@ -130,6 +130,7 @@ int mlora_pool_gather(const int32_t *tok_adapter, int T, const int32_t *page_tbl
     }
     if (!per_tok && !grouped) return MLORA_OK;
     mlora::GatherArgs a;
+    memset(&a, 0, sizeof(a));
     a.tok_adapter = tok_adapter; a.page_tbl = page_tbl; a.rank = rank; a.scaling = scaling;
     a.T = T; a.n_adapters = n_adapters; a.max_pages = max_pages > 0 ? max_pages : 1;
     a.page_rows = page_rows > 0 ? page_rows : 1; a.group = grouped ? group : 1;
@@ -430,6 +431,116 @@ int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const voi
     a.tok_adapter = nullptr; a.tok_adapter64 = indices;
     a.T = T; a.n_proj = 1; a.accumulate = 1;
     rc = mlora::launch_bgmv(a, dtype, 1, r, true, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+// Plan buffer of the reference-layout decode call: perm, seg_start, seg_len, seg_adapter, chunk_start, chunk_len,
+// chunk_adapter (T int32 each, padded to 16 bytes), counters, then the work records.
+static int64_t ref_plan_words(int T) { return ((int64_t)T + 3) / 4 * 4; }
+
+int64_t mlora_reflayout_plan_bytes(int T)
+{
+    if (T <= 0) return 0;
+    return (7 * ref_plan_words(T) + MLORA_CNT_WORDS + (int64_t)MLORA_WORK_CAP(T) * MLORA_WORK_WORDS) * (int64_t)sizeof(int32_t);
+}
+
+static int32_t *ref_plan_work(void *plan, int T) { return static_cast<int32_t *>(plan) + 7 * ref_plan_words(T) + MLORA_CNT_WORDS; }
+
+static int ref_rank_ok(int r) { return r == 8 || r == 16 || r == 32 || r == 64; }
+
+int mlora_reflayout_plan(const int64_t *indices, int T, int N, int L, int r, int group, void *plan, int64_t plan_bytes,
+                         void *stream)
+{
+    if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
+    if (T == 0) return MLORA_OK;
+    if (!indices || !plan) return fail(MLORA_EINVAL, "NULL pointer");
+    if (T > MLORA_GATHER_MAX_T) return fail(MLORA_ERANGE, "T = %d exceeds MLORA_GATHER_MAX_T = %d", T, MLORA_GATHER_MAX_T);
+    if (N <= 0 || N > (1 << 18) || L <= 0) return fail(MLORA_ERANGE, "N must be in 1..262144 and L positive (got %d, %d)", N, L);
+    if (!ref_rank_ok(r)) return fail(MLORA_ERANGE, "the grouped reference-layout call needs rank 8, 16, 32 or 64 (got %d); mlora_bgmv_reflayout takes any rank", r);
+    if (group != 1 && group != 2 && group != 4) return fail(MLORA_EINVAL, "group must be 1, 2 or 4 (got %d)", group);
+    if ((int64_t)N * L * r > 0x7fffffffLL) return fail(MLORA_ERANGE, "pool has more than 2^31-1 rank rows");
+    if (!aligned16(plan)) return fail(MLORA_EALIGN, "plan buffer must be 16-byte aligned");
+    if (plan_bytes < mlora_reflayout_plan_bytes(T))
+        return fail(MLORA_ENOSPACE, "plan buffer holds %lld bytes, %lld needed", (long long)plan_bytes, (long long)mlora_reflayout_plan_bytes(T));
+    mlora::GatherArgs a;
+    memset(&a, 0, sizeof(a));
+    int32_t *ip = static_cast<int32_t *>(plan);
+    const int64_t w = ref_plan_words(T);
+    a.tok_adapter64 = indices;
+    a.T = T; a.n_adapters = N; a.max_pages = 1; a.page_rows = 1; a.group = group;
+    // rank row j of adapter a, relative to a layer's first row: a * L * r + j (wa_T_all is [N, L, r, hin])
+    a.dense_stride = (long long)L * r; a.n_rows_dense = (long long)(N - 1) * L * r + r;
+    a.uniform_rank = r; a.uniform_scale = 1.0f;
+    a.perm = ip; a.seg_start = ip + w; a.seg_len = ip + 2 * w; a.seg_adapter = ip + 3 * w;
+    a.chunk_start = ip + 4 * w; a.chunk_len = ip + 5 * w; a.chunk_adapter = ip + 6 * w; a.counters = ip + 7 * w;
+    a.n_pages = 1; a.work = ref_plan_work(plan, T); a.work_cap = MLORA_WORK_CAP(T);
+    const int rc = mlora::launch_gather(a, static_cast<hipStream_t>(stream));
+    if (rc) return fail(MLORA_ELAUNCH, "gather launch failed: %s", hipGetErrorString((hipError_t)rc));
+    return MLORA_OK;
+}
+
+int mlora_bgmv_reflayout_multi(int n_proj, void *const *y, const void *const *x, const void *const *wa_T_all,
+                               const void *const *wb_T_all, const int32_t *hin, const int32_t *hout, const void *plan,
+                               int T, int N, int L, int r, int layer_idx, float scale, int group, int dtype,
+                               int accumulate, void *workspace, int64_t workspace_bytes, void *stream)
+{
+    if (dtype != MLORA_F16 && dtype != MLORA_BF16) return fail(MLORA_EDTYPE, "dtype must be MLORA_F16 or MLORA_BF16 (got %d)", dtype);
+    if (n_proj < 1 || n_proj > MLORA_MAX_PROJ) return fail(MLORA_ERANGE, "n_proj must be in 1..%d (got %d)", MLORA_MAX_PROJ, n_proj);
+    if (T < 0) return fail(MLORA_EINVAL, "T must be >= 0 (got %d)", T);
+    if (T == 0) return MLORA_OK;
+    if (!y || !x || !wa_T_all || !wb_T_all || !hin || !hout || !plan) return fail(MLORA_EINVAL, "NULL pointer");
+    if (N <= 0 || L <= 0) return fail(MLORA_EINVAL, "N and L must be positive (got %d, %d)", N, L);
+    if (layer_idx < 0 || layer_idx >= L) return fail(MLORA_ERANGE, "layer_idx %d outside [0, %d)", layer_idx, L);
+    if (!ref_rank_ok(r)) return fail(MLORA_ERANGE, "the grouped reference-layout call needs rank 8, 16, 32 or 64 (got %d); mlora_bgmv_reflayout takes any rank", r);
+    if (group != 1 && group != 2 && group != 4) return fail(MLORA_EINVAL, "group must be 1, 2 or 4 (got %d)", group);
+    if ((int64_t)N * L * r > 0x7fffffffLL) return fail(MLORA_ERANGE, "pool has more than 2^31-1 rank rows");
+    if (!aligned16(plan)) return fail(MLORA_EALIGN, "plan buffer must be 16-byte aligned");
+    mlora::BgmvArgs a;
+    memset(&a, 0, sizeof(a));
+    mlora::PoolView &pv = a.pool;
+    pv.n_adapters = N; pv.max_pages = 1; pv.page_shift = 0;
+    pv.uniform_rank = r; pv.uniform_scale = scale;
+    pv.a_dense_stride = (long long)L * r;
+    pv.n_rows_a = (long long)(N - 1) * L * r + r;
+    int max_hin = 0, max_hout = 0;
+    for (int p = 0; p < n_proj; p++) {
+        if (!y[p] || !x[p] || !wa_T_all[p] || !wb_T_all[p]) return fail(MLORA_EINVAL, "projection %d: NULL device pointer", p);
+        int rc = check_dims(hin[p], hout[p]);
+        if (rc) return rc;
+        a.y[p] = y[p]; a.x[p] = x[p];
+        a.a_rows[p] = static_cast<const uint16_t *>(wa_T_all[p]) + (size_t)layer_idx * r * hin[p];
+        a.b_rows[p] = static_cast<const uint16_t *>(wb_T_all[p]) + (size_t)layer_idx * hout[p] * r;
+        if (!aligned16(a.y[p]) || !aligned16(a.x[p]) || !aligned16(a.a_rows[p]) || !aligned16(a.b_rows[p]))
+            return fail(MLORA_EALIGN, "projection %d: device pointers must be 16-byte aligned", p);
+        a.hin[p] = hin[p]; a.hout[p] = hout[p];
+        max_hin = hin[p] > max_hin ? hin[p] : max_hin;
+        max_hout = hout[p] > max_hout ? hout[p] : max_hout;
+    }
+    a.b_transposed = 1; a.ref_layers = L;
+    a.tok_adapter = nullptr; a.tok_adapter64 = nullptr;
+    a.work = ref_plan_work(const_cast<void *>(plan), T); a.work_cap = MLORA_WORK_CAP(T);
+    {
+        const int64_t segs = T < N ? T : N;
+        const int64_t bound = ((int64_t)(T + group - 1) / group + segs + 1 + 7) / 8 * 8;
+        a.items_cap = bound < a.work_cap ? (int)bound : a.work_cap;
+    }
+    a.T = T; a.n_proj = n_proj; a.accumulate = accumulate ? 1 : 0;
+    const int64_t need = mlora_bgmv_workspace_bytes(n_proj, T, max_hin, r);
+    if (!workspace || !aligned16(workspace)) return fail(MLORA_EALIGN, "workspace must be a 16-byte aligned device pointer");
+    if (workspace_bytes < need) return fail(MLORA_ENOSPACE, "workspace holds %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
+    a.vws = static_cast<float *>(workspace);
+    int ksc, nte;
+    mlora::bgmv_split_slices(r, &ksc, &nte);
+    a.ks_max = (max_hin + ksc * 8 - 1) / (ksc * 8);
+    a.cs_max = (max_hout + nte * 8 - 1) / (nte * 8);
+    int sh = 0, ex = 0;
+    for (int p = 0; p < n_proj; p++) {
+        sh += (hin[p] + ksc * 8 - 1) / (ksc * 8);
+        ex += (hout[p] + nte * 8 - 1) / (nte * 8);
+        a.sh_end[p] = sh; a.ex_end[p] = ex;
+    }
+    const int rc = mlora::launch_bgmv_split(a, dtype, group, r, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "bgmv launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
 }

@@ -50,6 +50,8 @@ struct BgmvArgs {
     int T;
     int n_proj;
     int accumulate;
+    int b_transposed;              // two-launch form on the reference layout: b_rows[p] is [n_adapters, ref_layers, hout, rank] (this layer's
+    int ref_layers;                //   block first), adapter a's [hout, rank] block starts a * ref_layers * hout * rank elements in
     float *vws;                    // two-launch form: partial sums [n_proj, T, ks_max, rank stride] (else nullptr)
     int ks_max;                    // shrink slices of the widest hin (stride of the partial sums)
     int cs_max;                    // expand slices of the widest hout
@@ -82,10 +84,15 @@ struct AssistArgs {
 };
 
 struct GatherArgs {
-    const int32_t *tok_adapter;
-    const int32_t *page_tbl;
-    const int32_t *rank;
-    const float *scaling;
+    const int32_t *tok_adapter;    // [T] int32, or nullptr when tok_adapter64 is used
+    const int64_t *tok_adapter64;  // [T] int64 (the reference's index vector); an id outside [0, n_adapters) means no adapter
+    const int32_t *page_tbl;       // nullptr: dense pool, rank row j of adapter a is row a * dense_stride + j
+    const int32_t *rank;           // nullptr: every adapter has uniform_rank
+    const float *scaling;          // nullptr: every adapter has uniform_scale
+    long long dense_stride;
+    long long n_rows_dense;        // rows a dense slab holds (bounds the recorded rows)
+    int uniform_rank;
+    float uniform_scale;
     int T, n_adapters, max_pages, page_rows, group;
     long long n_pages;             // pages in a rows slab (bounds the recorded rows)
     int32_t *work;                 // [work_cap * WORK_WORDS] decode work records, or nullptr
@@ -172,7 +179,7 @@ struct GemmLoraArgs {
 
 // launchers (defined next to their kernels); return hipError_t as int
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
-int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);
+int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);   // a.b_transposed: max_rank is the pool's rank (8, 16, 32 or 64)
 int bgmv_split_rank_stride(int max_rank);
 void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);

@@ -18,6 +18,28 @@ constexpr int GATHER_NT_MAX = 1024;
 constexpr int GATHER_MAX_T = 8192;
 constexpr int TOK_BITS = 13;                 // token id field of the sort key
 
+// Adapter id of token i as the kernels see it: negative = none, >= n_adapters = out of range (counted, then none).
+// An int64 id (the reference's index vector) outside [0, n_adapters) is "none" on either side.
+__device__ __forceinline__ int gather_adapter(const GatherArgs &g, int i)
+{
+    if (g.tok_adapter) return g.tok_adapter[i];
+    const long long a = g.tok_adapter64[i];
+    return a < 0 ? -1 : (a >= g.n_adapters ? g.n_adapters : (int)a);
+}
+__device__ __forceinline__ int gather_rank(const GatherArgs &g, int a) { return g.rank ? g.rank[a] : g.uniform_rank; }
+__device__ __forceinline__ float gather_scale(const GatherArgs &g, int a) { return g.scaling ? g.scaling[a] : g.uniform_scale; }
+// Row (in a rows slab) of rank row j of adapter a, -1 if it does not exist.
+__device__ __forceinline__ int gather_row(const GatherArgs &g, int a, int j)
+{
+    if (!g.page_tbl) {
+        const long long row = (long long)a * g.dense_stride + j;
+        return row < g.n_rows_dense ? (int)row : -1;
+    }
+    if (j / g.page_rows >= g.max_pages) return -1;
+    const int pg = g.page_tbl[(long long)a * g.max_pages + j / g.page_rows];
+    return (pg >= 0 && pg < g.n_pages) ? pg * g.page_rows + j % g.page_rows : -1;
+}
+
 // Inclusive scan over the block's per-thread values; op = 0 sum, 1 max, 2 min.
 template <int OP>
 __device__ __forceinline__ int scan_op(int a, int b)
@@ -58,7 +80,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         const long long total = (long long)g.T * g.max_pages;
         if (idx >= total) return;
         const int t = (int)(idx / g.max_pages), pg = (int)(idx - (long long)t * g.max_pages);
-        int a = g.tok_adapter[t];
+        int a = gather_adapter(g, t);
         if (a >= g.n_adapters) a = -1;
         int r = 0;
         float s = 0.f;
@@ -95,7 +117,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         uint32_t key = 0xffffffffu;
         bool valid = false, bad = false;
         if (i < T) {
-            const int a = g.tok_adapter[i];
+            const int a = gather_adapter(g, i);
             bad = a >= g.n_adapters;
             valid = a >= 0 && !bad;
             key = ((valid ? (uint32_t)a : sentinel) << TOK_BITS) | (uint32_t)i;
@@ -207,7 +229,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
                 if (g.work) {
                     int rk = 0;
                     float sc = 0.f;
-                    if (real) { rk = g.rank[ad[e]]; rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); sc = g.scaling[ad[e]]; }
+                    if (real) { rk = gather_rank(g, ad[e]); rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); sc = gather_scale(g, ad[e]); }
                     s_chdr[ch_idx] = i | (len << TOK_BITS) | (rk << (TOK_BITS + 4));
                     s_cscale[ch_idx] = sc;
                 }
@@ -278,11 +300,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
                             const int j = j0 + e;
-                            rr[e] = -1;
-                            if (a >= 0 && j < rk && j / g.page_rows < g.max_pages) {
-                                const int pg = g.page_tbl[(long long)a * g.max_pages + j / g.page_rows];
-                                if (pg >= 0 && pg < g.n_pages) rr[e] = pg * g.page_rows + j % g.page_rows;
-                            }
+                            rr[e] = (a >= 0 && j < rk) ? gather_row(g, a, j) : -1;
                         }
                         v = make_int4(rr[0], rr[1], rr[2], rr[3]);
                     }
@@ -298,20 +316,16 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
             if ((b >> 3) < per_xcd && c < n_chunks) {
                 const int start = g.chunk_start[c], len = g.chunk_len[c], a = g.chunk_adapter[c];
                 int rk = 0;
-                if (a >= 0) { rk = g.rank[a]; rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); }
+                if (a >= 0) { rk = gather_rank(g, a); rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); }
                 if (w == 0) val = len;
                 else if (w == 1) val = a;
                 else if (w == 2) val = rk;
-                else if (w == 3) val = a >= 0 ? __builtin_bit_cast(int, g.scaling[a]) : 0;
+                else if (w == 3) val = a >= 0 ? __builtin_bit_cast(int, gather_scale(g, a)) : 0;
                 else if (w < 12) val = (w - 4) < len ? (int)(s_key[start + (w - 4)] & ((1u << TOK_BITS) - 1u)) : -1;
                 else if (w < WORK_ROWS_AT) val = 0;
                 else {
                     const int j = w - WORK_ROWS_AT;
-                    val = -1;
-                    if (a >= 0 && j < rk && j / g.page_rows < g.max_pages) {
-                        const int pg = g.page_tbl[(long long)a * g.max_pages + j / g.page_rows];
-                        if (pg >= 0 && pg < g.n_pages) val = pg * g.page_rows + j % g.page_rows;
-                    }
+                    val = (a >= 0 && j < rk) ? gather_row(g, a, j) : -1;
                 }
             }
             g.work[idx] = val;

@@ -53,6 +53,10 @@ SIGNATURES = {
     "mlora_bgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i64,
                           _i32, _i32, _i32, _vp]),
     "mlora_bgmv_reflayout": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp]),
+    "mlora_reflayout_plan_bytes": (_i64, [_i32]),
+    "mlora_reflayout_plan": (_i32, [_vp, _i32, _i32, _i32, _i32, _i32, _vp, _i64, _vp]),
+    "mlora_bgmv_reflayout_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32,
+                                          _i32, _i32, _vp, _i64, _vp]),
     "mlora_sgmv_workspace_bytes": (_i64, [_i32, _i32]),
     "mlora_sgmv": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                           _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),

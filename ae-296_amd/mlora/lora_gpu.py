@@ -49,6 +49,12 @@ class Lora_GPU:
         self.select_inds = [torch.randint(0, hi, (i + 1,), device=self.device, generator=self._gen)
                             for i in range(self.batch_size)]
         self._workspace = None
+        self._plan = None          # grouping of the current decode batch by adapter, and what it was made from
+        self._plan_key = None
+        self._qkv = None           # q, k, v deltas of the last decode input, and what they were computed from
+        self._qkv_key = None
+        self._ids = None           # int64 copy of the last int32 lora_ids
+        self._ids_key = None
 
     def _rand(self, n, rows, cols):
         """[n, L, rows, cols] * 0.001, stored transposed and contiguous as the reference does."""
@@ -57,6 +63,57 @@ class Lora_GPU:
         return w.to(self.dtype).transpose(-1, -2).contiguous()
 
     # ------------------------------------------------------------------ apply
+    def _indices(self, bsz, lora_ids, device):
+        # The reference drops the request's adapter ids (``infer_state.lora_ids``, built at
+        # pre_process.py:50,100) and applies a random stand-in; pass ``lora_ids`` to use the real ones.
+        if lora_ids is None:
+            return self.select_inds[bsz - 1]
+        if lora_ids.numel() != bsz:
+            raise ValueError("lora_ids must hold one adapter slot per row of x")
+        if lora_ids.dtype == torch.int64 and lora_ids.device == device:
+            return lora_ids
+        # int32 ids (pre_process.py:100) are widened once per distinct tensor contents, so that the three calls of a
+        # layer (and the layers of a step) see one index vector
+        key = (lora_ids.data_ptr(), lora_ids._version, str(lora_ids.device), lora_ids.dtype)
+        if self._ids_key != key:
+            self._ids, self._ids_key = lora_ids.to(device=device, dtype=torch.int64), key
+        return self._ids
+
+    def plan_decode(self, bsz, lora_ids=None):
+        """Group the decode batch by adapter (one gather launch).  Called by ``invoke_one_layer_qkv`` when the index
+        vector is not the one the current plan was made from; a serving loop calls it once per step."""
+        device = self.q_down.device
+        cur_inds = self._indices(bsz, lora_ids, device)
+        reuse = self._plan if (self._plan is not None and self._plan.T == bsz) else None
+        self._plan = ops.plan_decode_ref(cur_inds, self.batch_size, self.n_layers, self.lora_rank, out=reuse)
+        self._plan_key = (cur_inds.data_ptr(), cur_inds._version, bsz)
+        self._qkv_key = None
+        return self._plan
+
+    def invoke_one_layer_qkv(self, x, layer_id, lora_ids=None):
+        """The q, k and v deltas of one decode layer in one call pair (the reference makes three
+        ``add_lora_bgmv`` calls with a ``torch.zeros`` each, lora_gpu.py:137-138,149-150,161-162): returns
+        ``(q_lora, k_lora, v_lora)``, each ``[bsz, hidden / tp]``."""
+        bsz = x.shape[0]
+        if not ops.ref_rank_supported(self.lora_rank):
+            return tuple(self._invoke_single(n, x, layer_id, lora_ids) for n in "qkv")
+        cur_inds = self._indices(bsz, lora_ids, x.device)
+        if self._plan is None or self._plan_key != (cur_inds.data_ptr(), cur_inds._version, bsz):
+            self.plan_decode(bsz, cur_inds)
+        if not x.is_contiguous():
+            x = x.contiguous()
+        ys = [torch.empty(bsz, self.output_size, device=x.device, dtype=x.dtype) for _ in range(3)]
+        ops.add_lora_bgmv_multi(ys, [x, x, x], [self.q_down, self.k_down, self.v_down], [self.q_up, self.k_up, self.v_up],
+                                self._plan, layer_id, 1.0, accumulate=False)
+        return tuple(ys)
+
+    def _invoke_single(self, name, x, layer_id, lora_ids):
+        bsz = x.shape[0]
+        cur_inds = self._indices(bsz, lora_ids, x.device)
+        y = torch.zeros(bsz, self.output_size, device=x.device, dtype=x.dtype)
+        ops.add_lora_bgmv(y, x, getattr(self, f"{name}_down"), getattr(self, f"{name}_up"), cur_inds, layer_id, 1)
+        return y
+
     def _invoke(self, name, x, layer_id, prefill, lora_ids=None):
         bsz = x.shape[0]
         if prefill:
@@ -69,17 +126,18 @@ class Lora_GPU:
             if self._workspace is None or self._workspace.numel() < need:
                 self._workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
             return ops.lora_prefill_ref(x, down, up, layer_id, workspace=self._workspace)
-        # The reference drops the request's adapter ids (``infer_state.lora_ids``, built at
-        # pre_process.py:50,100) and applies a random stand-in; pass ``lora_ids`` to use the real ones.
-        if lora_ids is None:
-            cur_inds = self.select_inds[bsz - 1]
-        else:
-            if lora_ids.numel() != bsz:
-                raise ValueError("lora_ids must hold one adapter slot per row of x")
-            cur_inds = lora_ids.to(device=x.device, dtype=torch.int64)
-        y = torch.zeros(bsz, self.output_size, device=x.device, dtype=x.dtype)
-        ops.add_lora_bgmv(y, x, getattr(self, f"{name}_down"), getattr(self, f"{name}_up"), cur_inds, layer_id, 1)
-        return y
+        if not ops.ref_rank_supported(self.lora_rank):
+            return self._invoke_single(name, x, layer_id, lora_ids)
+        # ``_get_qkv`` asks for q, k and v of the same input one after the other
+        # (transformer_layer_infer.py:109-111): the first of the three calls computes all of them in one call pair,
+        # the other two are answered from that result as long as the input tensor, its contents (torch's version
+        # counter), the layer and the index vector are the same.
+        cur_inds = self._indices(bsz, lora_ids, x.device)
+        key = (x.data_ptr(), x._version, tuple(x.shape), layer_id, cur_inds.data_ptr(), cur_inds._version)
+        if self._qkv_key != key or name not in self._qkv:
+            q, k, v = self.invoke_one_layer_qkv(x, layer_id, cur_inds)
+            self._qkv, self._qkv_key = {"q": q, "k": k, "v": v}, key
+        return self._qkv.pop(name)
 
     def invoke_one_layer_q(self, x, layer_id, prefill=False, lora_ids=None):
         return self._invoke("q", x, layer_id, prefill, lora_ids)
@@ -93,6 +151,7 @@ class Lora_GPU:
     # ------------------------------------------------------------------ slot management
     def prepare_lora_prefill(self, batch_size):
         """lora_gpu.py:190-200: fresh random prefill adapters, one slot per request."""
+        self._qkv_key = None
         for name in ("q", "k", "v"):
             setattr(self, f"{name}_down_prefill", self._rand(batch_size, self.in_size, self.lora_rank))
             setattr(self, f"{name}_up_prefill", self._rand(batch_size, self.lora_rank, self.output_size))
@@ -100,6 +159,7 @@ class Lora_GPU:
     def merge_lora_prefill(self, bsz, re_inds=None):
         """lora_gpu.py:202-217: copy the first bsz prefill slots into decode slots (random targets
         in the reference; pass re_inds to choose them)."""
+        self._qkv_key = None                    # weights change: results computed from the old ones are not served again
         if re_inds is None:
             re_inds = np.random.randint(0, self.batch_size, size=bsz)
         for idx, re_ind in enumerate(re_inds):
@@ -114,6 +174,7 @@ class Lora_GPU:
         is applied to the adapter axis here."""
         if running_bsz <= 0:
             return
+        self._qkv_key = None
         if chosen is None:
             chosen = np.random.randint(0, running_bsz, size=len(rm_ids))
         for rm_id in chosen:

@@ -148,16 +148,24 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
     if tok_adapter.dtype != torch.int32:
         raise TypeError("tok_adapter must be int32")
     T = tok_adapter.numel()
-    yv, xv, av, bv, hi, ho = _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
-    for i, p in enumerate(projs):
-        hin, hout = pool.projections[p]
+    # the slab pointers and widths of a (layer, projections) pair never change: their argument arrays are kept
+    key = (layer, tuple(projs))
+    cached = pool._call_args.get(key)
+    if cached is None:
+        av, bv, hi, ho = _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
+        for i, p in enumerate(projs):
+            hi[i], ho[i] = pool.projections[p]
+            av[i], bv[i] = pool.slab_ptrs(layer, p)
+        cached = pool._call_args[key] = (av, bv, hi, ho, max(hi[i] for i in range(n)))
+    av, bv, hi, ho, max_hin = cached
+    yv, xv = _VoidArr(), _VoidArr()
+    for i in range(n):
         if xs[i].dtype != pool.dtype or ys[i].dtype != pool.dtype:
             raise TypeError(f"x and y must have the pool dtype {pool.dtype}")
-        if tuple(xs[i].shape) != (T, hin) or tuple(ys[i].shape) != (T, hout):
-            raise ValueError(f"projection {p}: expected x [{T}, {hin}] and y [{T}, {hout}], "
+        if xs[i].shape[0] != T or xs[i].shape[1] != hi[i] or ys[i].shape[0] != T or ys[i].shape[1] != ho[i] or xs[i].dim() != 2 or ys[i].dim() != 2:
+            raise ValueError(f"projection {projs[i]}: expected x [{T}, {hi[i]}] and y [{T}, {ho[i]}], "
                              f"got {tuple(xs[i].shape)} and {tuple(ys[i].shape)}")
-        a_ptr, b_ptr = pool.slab_ptrs(layer, p)
-        yv[i], xv[i], av[i], bv[i], hi[i], ho[i] = ys[i].data_ptr(), xs[i].data_ptr(), a_ptr, b_ptr, hin, hout
+        yv[i], xv[i] = ys[i].data_ptr(), xs[i].data_ptr()
     pool.sync()
     if plan is not None and plan.T != T:
         raise ValueError("plan was built for a different batch size")
@@ -167,7 +175,7 @@ def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPo
         raise ValueError("the two-launch form needs a plan")
     ws, ws_bytes = None, 0
     if not fused:
-        ws_bytes = _ext.lib().mlora_bgmv_workspace_bytes(n, T, max(hi[i] for i in range(n)), pool.max_rank)
+        ws_bytes = _ext.lib().mlora_bgmv_workspace_bytes(n, T, max_hin, pool.max_rank)
         if plan.vws is None or plan.vws.numel() < ws_bytes:
             plan.vws = torch.empty(ws_bytes, dtype=torch.uint8, device=tok_adapter.device)
         ws = plan.vws
@@ -206,6 +214,90 @@ def add_lora_bgmv(y: torch.Tensor, x: torch.Tensor, wa_T_all: torch.Tensor, wb_T
     rc = _ext.lib().mlora_bgmv_reflayout(y.data_ptr(), x.data_ptr(), wa_T_all.data_ptr(), wb_T_all.data_ptr(),
                                          indicies.data_ptr(), T, N, L, r, hin, hout, layer_idx, float(scale), dt,
                                          _ext.current_stream_ptr())
+    _ext.check(rc)
+
+
+@dataclass
+class RefDecodePlan:
+    """Grouping of one decode batch by adapter for the reference-layout calls (written by ``mlora_reflayout_plan``)."""
+    indicies: torch.Tensor         # int64 [T]
+    group: int
+    N: int
+    L: int
+    r: int
+    buf: torch.Tensor              # uint8: perm, segments, chunks, counters, work records
+    vws: Optional[torch.Tensor] = None
+
+    @property
+    def T(self) -> int:
+        return self.indicies.numel()
+
+
+def ref_rank_supported(r: int) -> bool:
+    """Ranks the grouped reference-layout call takes (the plain ``add_lora_bgmv`` takes any rank up to 64)."""
+    return r in (8, 16, 32, 64)
+
+
+def plan_decode_ref(indicies: torch.Tensor, N: int, L: int, r: int, group: Optional[int] = None,
+                    out: Optional[RefDecodePlan] = None) -> RefDecodePlan:
+    """Group a decode batch by adapter for ``add_lora_bgmv_multi``: once per step, the plan serves every layer and
+    projection that uses this index vector on pools of N adapters, L layers and rank r.  Pass `out` to reuse a
+    plan's buffers (no allocation; safe under graph capture)."""
+    _need_cuda(indicies)
+    _need_contig(indicies)
+    if indicies.dtype != torch.int64:
+        raise TypeError("indicies must be int64 (as torch.randint produces at lora_gpu.py:120)")
+    T = indicies.numel()
+    if group is None:
+        group = out.group if out is not None else min(4, default_group(T))
+    lib = _ext.lib()
+    if out is None:
+        out = RefDecodePlan(indicies, group, N, L, r,
+                            torch.empty(max(16, lib.mlora_reflayout_plan_bytes(T)), dtype=torch.uint8, device=indicies.device))
+    else:
+        if out.T != T or (out.N, out.L, out.r) != (N, L, r):
+            raise ValueError("the plan to reuse was made for another batch size or pool")
+        out.indicies, out.group = indicies, group
+    _ext.check(lib.mlora_reflayout_plan(indicies.data_ptr(), T, N, L, r, group, out.buf.data_ptr(), out.buf.numel(),
+                                        _ext.current_stream_ptr()))
+    return out
+
+
+def add_lora_bgmv_multi(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], was: Sequence[torch.Tensor],
+                        wbs: Sequence[torch.Tensor], plan: RefDecodePlan, layer_idx: int, scale: float,
+                        accumulate: bool = True) -> None:
+    """``punica.ops.add_lora_bgmv`` for several projections of one layer in one call pair, on the reference's pool
+    layout in place: ``ys[p][i] (+)= xs[p][i] @ was[p][idx[i], layer].T @ wbs[p][idx[i], layer].T * scale`` with
+    was[p] [N, L, r, Hin], wbs[p] [N, L, Hout, r] and idx the index vector the plan was made from
+    (``lora_gpu.py:137-138,149-150,161-162`` in one go).  ``accumulate=False`` defines ys as the delta alone
+    (zeros for indices outside the pool), which saves the ``torch.zeros`` of ``lora_gpu.py:137``."""
+    n = len(ys)
+    if not (len(xs) == len(was) == len(wbs) == n) or not 1 <= n <= _ext.MAX_PROJ:
+        raise ValueError(f"need 1..{_ext.MAX_PROJ} projections with one y, x, wa and wb each")
+    _need_cuda(*ys, *xs, *was, *wbs)
+    _need_contig(*ys, *xs, *was, *wbs)
+    T = plan.T
+    yv, xv, av, bv, hi, ho = _VoidArr(), _VoidArr(), _VoidArr(), _VoidArr(), _IntArr(), _IntArr()
+    dt = ys[0].dtype
+    for i in range(n):
+        if was[i].dim() != 4 or wbs[i].dim() != 4:
+            raise ValueError("wa_T_all must be [N, L, r, Hin] and wb_T_all [N, L, Hout, r]")
+        N, L, r, hin = was[i].shape
+        N2, L2, hout, r2 = wbs[i].shape
+        if (N2, L2, r2) != (N, L, r) or (N, L, r) != (plan.N, plan.L, plan.r):
+            raise ValueError("pool tensors disagree with each other or with the plan on N, L or r")
+        if tuple(xs[i].shape) != (T, hin) or tuple(ys[i].shape) != (T, hout):
+            raise ValueError("x must be [B, Hin] and y [B, Hout] for the plan's batch")
+        if not (ys[i].dtype == xs[i].dtype == was[i].dtype == wbs[i].dtype == dt):
+            raise TypeError("y, x and the pools must share one 16-bit dtype")
+        yv[i], xv[i], av[i], bv[i], hi[i], ho[i] = ys[i].data_ptr(), xs[i].data_ptr(), was[i].data_ptr(), wbs[i].data_ptr(), hin, hout
+    lib = _ext.lib()
+    ws_bytes = lib.mlora_bgmv_workspace_bytes(n, T, max(hi[i] for i in range(n)), plan.r)
+    if plan.vws is None or plan.vws.numel() < ws_bytes:
+        plan.vws = torch.empty(ws_bytes, dtype=torch.uint8, device=ys[0].device)
+    rc = lib.mlora_bgmv_reflayout_multi(n, yv, xv, av, bv, hi, ho, plan.buf.data_ptr(), T, plan.N, plan.L, plan.r, layer_idx,
+                                        float(scale), plan.group, _ext.dtype_code(dt), int(accumulate),
+                                        plan.vws.data_ptr(), plan.vws.numel(), _ext.current_stream_ptr())
     _ext.check(rc)
 
 

@@ -60,6 +60,7 @@ class AdapterPool:
         self.scaling = torch.zeros(n_slots, dtype=torch.float32, device=self.device)
         self._free = list(range(n_pages - 1, -1, -1))
         self._dirty = False
+        self._call_args = {}       # (layer, projections) -> argument arrays of the decode call (kept by ops.bgmv)
 
     # ------------------------------------------------------------------ page table
     def allocate(self, slot: int, rank: int, scaling: float, pages: Sequence[int] | None = None) -> np.ndarray:

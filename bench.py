@@ -447,6 +447,8 @@ def bench_reflayout(args, dev, steps, warmup, min_ms=0.0):
     batched = getattr(gpu, "invoke_one_layer_qkv", None) if not args.fused else None    # --fused: one call per projection
 
     def step():
+        if batched is not None:
+            gpu.plan_decode(T, ids)                          # once per step, as a serving loop would
         for l in range(L):
             if batched is not None:
                 batched(xs[l], l, lora_ids=ids)
@@ -462,6 +464,23 @@ def bench_reflayout(args, dev, steps, warmup, min_ms=0.0):
     run = graph_of(step)
     greps = reps_for(run, steps, min_ms) if min_ms else steps
     t = timed(run, greps, warmup)
+    # the paged call on the same batch (same index vector, q/k/v, rank-16 adapters on pool pages), for the ratio
+    wl = workloads.make_decode("ref_cmp", {p: (H, H) for p in "qkv"}, L, T, N, [r], 1.0, seed=1002, device=dev,
+                               tok_adapter=ids.cpu().numpy().astype(np.int32))
+    tok32 = torch.from_numpy(wl.tok_adapter).to(dev)
+    pplan = mlora.plan_decode(tok32, wl.pool, group=4)
+    pys = [[torch.empty(T, H, device=dev, dtype=torch.float16) for _ in range(3)] for _ in range(L)]
+
+    def paged_step():
+        mlora.plan_decode(tok32, wl.pool, group=4, out=pplan)
+        for l in range(L):
+            mlora.bgmv(pys[l], [xs[l]] * 3, wl.pool, l, ["q", "k", "v"], tok32, plan=pplan, accumulate=False, fused=False)
+
+    paged_step()
+    torch.cuda.synchronize()
+    prun = graph_of(paged_step)
+    tp = timed(prun, reps_for(prun, steps, min_ms) if min_ms else steps, warmup)
+    del wl, pplan, pys
     uniq = np.unique(ids.cpu().numpy())
     # x is read once for q, k, v; y is written, not read (the call starts from zeros); indices are int64
     alg = T * H * 2 + 3 * T * H * 2 + 3 * len(uniq) * r * (H + H) * 2 + 8 * T
@@ -474,7 +493,8 @@ def bench_reflayout(args, dev, steps, warmup, min_ms=0.0):
             "config": {"workload": "reference layout, config-2 size: q/k/v 4096->4096, 256 tokens, 64 rank-16 adapters, Zipf(1.0), "
                                    "fp16, pool [N,L,r,Hin] / [N,L,Hout,r], int64 indices", "layers": L, "tokens": T,
                        "form": "one q/k/v call per layer" if batched is not None else "one call per projection", "hip_graph": True,
-                       "eager_ms_per_step": eager["ms"], "eager_spread": {k: eager[k] for k in ("p10", "p50", "p90")}},
+                       "eager_ms_per_step": eager["ms"], "eager_spread": {k: eager[k] for k in ("p10", "p50", "p90")},
+                       "paged_call_same_batch_ms_per_step": tp["ms"], "ratio_to_paged_call": t["ms"] / tp["ms"]},
             "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                          "traffic": None, "traffic_source": None, "kernel": "one layer's q/k/v calls on the reference layout",
                          "launch_us": launch_us, "algorithmic_bytes_per_launch": alg},
@@ -801,7 +821,7 @@ def leg_of(line):
     keep = {k: line[k] for k in ("metric", "value", "unit", "ms_per_step", "ms_per_step_spread", "steps", "dtype")}
     keep["workload"] = line["config"]["workload"]
     keep["form"] = line["config"].get("form")
-    for k in ("eager_ms_per_step", "library_gemm_then_sgmv_ms", "speedup_over_library_gemm_then_sgmv", "tokens", "adapters_touched",
+    for k in ("eager_ms_per_step", "paged_call_same_batch_ms_per_step", "ratio_to_paged_call", "library_gemm_then_sgmv_ms", "speedup_over_library_gemm_then_sgmv", "tokens", "adapters_touched",
               "steps_in_trace", "adapters_touched_per_step", "swap_ins"):
         if k in line["config"]:
             keep[k] = line["config"][k]

@@ -236,6 +236,28 @@ int mlora_bgmv_reflayout(void *y, const void *x, const void *wa_T_all, const voi
                          int layer_idx, float scale, int dtype, void *stream);
 
 /*
+ * The same call in the grouped two-launch form, for several projections of one layer that use the same index vector
+ * (the reference calls add_lora_bgmv three times per layer, for q, k and v: lora_gpu.py:137-138,149-150,161-162).
+ *   mlora_reflayout_plan groups the tokens of a batch by adapter once (the plan serves every layer and projection
+ *     of the step): indices int64 [T]; plan = device buffer of mlora_reflayout_plan_bytes(T) bytes.  An index outside
+ *     [0, N) means "no adapter" for that token.
+ *   mlora_bgmv_reflayout_multi: y_p[t] = (accumulate ? y_p[t] : 0) + scale * (x_p[t] . wa_p[idx[t], layer]^T) . wb_p[idx[t], layer]^T
+ *     for projection p < n_proj, wa_p [N, L, r, hin_p], wb_p [N, L, hout_p, r] in place (nothing is copied or
+ *     transposed); y, x, wa_T_all, wb_T_all, hin, hout are HOST arrays of n_proj entries.  accumulate = 0 writes
+ *     zeros for tokens without adapter, so the caller needs no torch.zeros before the call (lora_gpu.py:137).
+ *     workspace: mlora_bgmv_workspace_bytes(n_proj, T, max hin, r) bytes; group as given to the plan (1, 2 or 4).
+ * Rank 8, 16, 32 or 64 (MLORA_ERANGE otherwise; mlora_bgmv_reflayout takes any rank up to 64).
+ */
+int64_t mlora_reflayout_plan_bytes(int T);
+int mlora_reflayout_plan(const int64_t *indices, int T, int N, int L, int r, int group,
+                         void *plan, int64_t plan_bytes, void *stream);
+int mlora_bgmv_reflayout_multi(int n_proj, void *const *y, const void *const *x,
+                               const void *const *wa_T_all, const void *const *wb_T_all,
+                               const int32_t *hin, const int32_t *hout, const void *plan,
+                               int T, int N, int L, int r, int layer_idx, float scale, int group,
+                               int dtype, int accumulate, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * Prefill (SGMV): tokens are packed contiguously per segment; segment s covers tokens
  * [seg_start[s], seg_start[s] + seg_len[s]) and uses adapter seg_adapter[s] (negative = none):
  *     y[t] = (accumulate ? y[t] : 0) + scaling[a] * (x[t] . A_a) . B_a

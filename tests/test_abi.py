@@ -98,5 +98,15 @@ def test_validation_errors_without_gpu():
     assert rc == _ext.MLORA_ENOSPACE
     rc = lib.mlora_bgmv_reflayout(one, one, one, one, one, 4, 8, 32, 16, 64, 64, 32, 1.0, 0, None)
     assert rc == _ext.MLORA_ERANGE                     # layer_idx == L
+    # grouped reference-layout call: ranks 8 / 16 / 32 / 64 only, plan buffer and workspace sizes checked
+    assert lib.mlora_reflayout_plan_bytes(256) == (7 * 256 + 8 + 256 * 80) * 4
+    assert lib.mlora_reflayout_plan(one, 10, 8, 2, 12, 4, one, 1 << 20, None) == _ext.MLORA_ERANGE
+    assert b"rank 8, 16, 32 or 64" in lib.mlora_last_error()
+    assert lib.mlora_reflayout_plan(one, 10, 8, 2, 16, 4, one, 64, None) == _ext.MLORA_ENOSPACE
+    assert lib.mlora_reflayout_plan(one, 10, 8, 2, 16, 8, one, 1 << 20, None) == _ext.MLORA_EINVAL
+    rc = lib.mlora_bgmv_reflayout_multi(1, P, P, P, P, H, H, one, 10, 8, 2, 16, 2, 1.0, 4, 0, 1, one, 1 << 20, None)
+    assert rc == _ext.MLORA_ERANGE                     # layer_idx == L
+    rc = lib.mlora_bgmv_reflayout_multi(1, P, P, P, P, H, H, one, 10, 8, 2, 16, 1, 1.0, 4, 0, 1, one, 16, None)
+    assert rc == _ext.MLORA_ENOSPACE
     rc = lib.mlora_prefill_reflayout(one, one, one, one, 2, 16, 4, 12, 64, 64, 0, 0, one, 1 << 30, None)
     assert rc == _ext.MLORA_ERANGE                     # rank not a multiple of 8

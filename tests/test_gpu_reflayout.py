@@ -35,6 +35,96 @@ def test_add_lora_bgmv_vs_oracle(N, L, r, hin, hout, T, layer, scale, dtype):
     assert_close_bits(torch_to_bits(y), want, dtype)
 
 
+@pytest.mark.parametrize("r,group,T,dtype", [(16, 4, 256, FP16), (8, 1, 33, FP16), (32, 2, 100, BF16), (64, 4, 70, FP16),
+                                             (16, 2, 5, BF16), (64, 1, 9, BF16)])
+def test_add_lora_bgmv_multi_vs_oracle(r, group, T, dtype):
+    """q, k, v of one layer in one call pair on the reference layout, in place: three pools, projections of different
+    widths, indices that repeat (grouped items) and some outside the pool, accumulate and delta forms."""
+    from mlora import add_lora_bgmv_multi, plan_decode_ref
+    rng = np.random.default_rng(r * 1000 + T)
+    N, L, layer, scale = 11, 3, 2, 0.5
+    shapes = [(512, 512), (512, 264), (1032, 2056)]            # q, k (narrower, tensor-parallel style), an odd-width pair
+    was = [bits_of((rng.standard_normal((N, L, r, hin)) * 0.05).astype(np.float32), dtype) for hin, _ in shapes]
+    wbs = [bits_of((rng.standard_normal((N, L, hout, r)) * 0.05).astype(np.float32), dtype) for _, hout in shapes]
+    idx = rng.integers(0, N, T).astype(np.int64)
+    idx[rng.random(T) < 0.4] = 3                                  # a hot adapter: several grouped items
+    bad = np.zeros(T, bool)
+    bad[::13] = True
+    idx_dev = idx.copy()
+    idx_dev[bad] = np.where(np.arange(T)[bad] % 2 == 0, -1, N + 2)
+    xs = [bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype) for hin, _ in shapes]
+    y0 = [bits_of(rng.standard_normal((T, hout)).astype(np.float32), dtype) for _, hout in shapes]
+    ids = torch.from_numpy(idx_dev).cuda()
+    plan = plan_decode_ref(ids, N, L, r, group=group)
+    wa_t = [bits_to_torch(w, dtype, "cuda") for w in was]
+    wb_t = [bits_to_torch(w, dtype, "cuda") for w in wbs]
+    x_t = [bits_to_torch(x, dtype, "cuda") for x in xs]
+    for accumulate in (True, False):
+        ys = [bits_to_torch(y, dtype, "cuda") if accumulate else
+              torch.full(y.shape, float("nan"), dtype=wa_t[0].dtype, device="cuda") for y in y0]
+        say(f"add_lora_bgmv_multi r={r} group={group} T={T} accumulate={accumulate}")
+        add_lora_bgmv_multi(ys, x_t, wa_t, wb_t, plan, layer, scale, accumulate=accumulate)
+        torch.cuda.synchronize()
+        for p in range(3):
+            base = y0[p].copy() if accumulate else np.zeros_like(y0[p])
+            want = base.copy()
+            orc.add_lora_bgmv_ref(want, xs[p], was[p], wbs[p], idx, layer, scale, dtype)
+            want[bad] = base[bad]                                  # an index outside the pool: no adapter
+            got = torch_to_bits(ys[p])
+            assert np.array_equal(got[bad], base[bad])
+            assert_close_bits(got, want, dtype, f"projection {p}")
+
+
+def test_add_lora_bgmv_multi_integer_inputs_bit_exact():
+    from mlora import add_lora_bgmv_multi, plan_decode_ref
+    rng = np.random.default_rng(77)
+    N, L, r, H, T = 6, 2, 16, 512, 45
+    wa = bits_of(rng.integers(-1, 2, (N, L, r, H)).astype(np.float32), FP16)
+    wb = bits_of(rng.integers(-1, 2, (N, L, H, r)).astype(np.float32), FP16)
+    idx = rng.integers(0, N, T).astype(np.int64)
+    x = bits_of((rng.integers(-2, 3, (T, H)) * (rng.random((T, H)) < 0.05)).astype(np.float32), FP16)
+    y0 = bits_of(rng.integers(-8, 9, (T, H)).astype(np.float32), FP16)
+    want = y0.copy()
+    orc.add_lora_bgmv_ref(want, x, wa, wb, idx, 1, 2.0, FP16)
+    assert np.abs(f32_of(want, FP16)).max() < 2048
+    plan = plan_decode_ref(torch.from_numpy(idx).cuda(), N, L, r, group=4)
+    y = bits_to_torch(y0, FP16, "cuda")
+    say("add_lora_bgmv_multi integer-valued inputs")
+    add_lora_bgmv_multi([y], [bits_to_torch(x, FP16, "cuda")], [bits_to_torch(wa, FP16, "cuda")], [bits_to_torch(wb, FP16, "cuda")],
+                        plan, 1, 2.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(torch_to_bits(y), want)
+
+
+def test_lora_gpu_qkv_in_one_call_pair_and_served_to_the_three_calls():
+    """invoke_one_layer_qkv against the fp32 expression; the reference's q, k, v calls on one input get the same bits,
+    computed once; a changed input, layer or weight set is computed afresh."""
+    cfg = dict(n_layers=3, batch_size=20, lora_rank=16, hidden_dim=1024, tp_degree=2, max_prefill_batch_size=2)
+    g = Lora_GPU(cfg, seed=5)
+    x = torch.randn(37 % 20 + 1, 1024, device="cuda", dtype=torch.float16)
+    bsz = x.shape[0]
+    ids = torch.randint(0, 20, (bsz,), device="cuda", dtype=torch.int32)
+    say("Lora_GPU.invoke_one_layer_qkv")
+    q, k, v = g.invoke_one_layer_qkv(x, 2, lora_ids=ids)
+    for name, got in zip("qkv", (q, k, v)):
+        down, up = getattr(g, f"{name}_down"), getattr(g, f"{name}_up")
+        want = torch.stack([x[i].float() @ down[ids[i], 2].float().t() @ up[ids[i], 2].float().t() for i in range(bsz)])
+        assert got.shape == (bsz, 512) and torch.allclose(got.float(), want, rtol=RTOL, atol=ATOL)
+    q1 = g.invoke_one_layer_q(x, 2, False, lora_ids=ids)
+    plan_after_q = g._plan_key
+    k1 = g.invoke_one_layer_k(x, 2, False, lora_ids=ids)
+    v1 = g.invoke_one_layer_v(x, 2, False, lora_ids=ids)
+    assert g._plan_key == plan_after_q                        # one plan, made before
+    assert torch.equal(q1, q) and torch.equal(k1, k) and torch.equal(v1, v)
+    x.mul_(2.0)                                                # same storage, new contents
+    q2 = g.invoke_one_layer_q(x, 2, False, lora_ids=ids)
+    assert not torch.equal(q2, q)
+    g.merge_lora_prefill(0)                                    # weights may have changed: nothing stale is served
+    k2 = g.invoke_one_layer_k(x, 2, False, lora_ids=ids)
+    want = torch.stack([x[i].float() @ g.k_down[ids[i], 2].float().t() @ g.k_up[ids[i], 2].float().t() for i in range(bsz)])
+    assert torch.allclose(k2.float(), want, rtol=RTOL, atol=ATOL)
+
+
 def test_add_lora_bgmv_bad_index_leaves_row_untouched():
     rng = np.random.default_rng(3)
     N, L, r, H, T = 4, 1, 8, 128, 6
