@@ -177,39 +177,46 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     int proj = 0;
     while (proj + 1 < p.n_proj && id.q >= p.sh_end[proj]) proj++;
     const int ks = id.q - (proj ? p.sh_end[proj - 1] : 0);
-    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
-    int ntok = rec[0];
-    if (ntok <= 0) return;
-    ntok = ntok < G ? ntok : G;
-    const int adapter = rec[1];
-    if (adapter < 0) return;
-    int r = rec[2];
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    int tok[G];
+    // A workgroup serves records id.b, id.b + stride, ...: the launch covers `rec_stride` records, not the
+    // host's upper bound on them (the records in use of one XCD residue are a prefix, so the first empty one ends
+    // the walk).  Most batches need one pass; what a grid over the whole bound would spend on dispatching
+    // workgroups of empty records is saved.
+    for (int b = id.b; b < p.items_cap; b += p.rec_stride_sh) {
+        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+        int ntok = rec[0];
+        if (ntok <= 0) break;
+        ntok = ntok < G ? ntok : G;
+        const int adapter = rec[1];
+        if (adapter < 0) continue;
+        int r = rec[2];
+        r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
+        int tok[G];
 #pragma unroll
-    for (int k = 0; k < G; k++) {
-        const int t = k < ntok ? rec[4 + k] : -1;
-        tok[k] = (t >= 0 && t < p.T) ? t : -1;
-    }
-    const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+        for (int k = 0; k < G; k++) {
+            const int t = k < ntok ? rec[4 + k] : -1;
+            tok[k] = (t >= 0 && t < p.T) ? t : -1;
+        }
+        const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
 
-    // r is uniform over the workgroup: a scalar branch, no divergence.  An item of a lower rank bucket
-    // takes F consecutive slices in one workgroup (the others of the F leave at once) and stores its sums
-    // in the slot of the first.
-    auto go = [&](auto nr_tag, auto f_tag) {
-        constexpr int NR = decltype(nr_tag)::value, F = decltype(f_tag)::value;
-        if (ks % F) return;
-        shrink_rows<DT, G, RMAX, KSC * F, NR, BIG>(p, rows, tok, r, proj, ks / F, ks, s_part);
-    };
-    using SF = SliceFactor<RMAX>;
-    if constexpr (RMAX >= 64) {
-        if (r > 32) { go(std::integral_constant<int, 16>{}, std::integral_constant<int, SF::F16>{}); return; }
+        // r is uniform over the workgroup: a scalar branch, no divergence.  An item of a lower rank bucket
+        // takes F consecutive slices in one workgroup (the others of the F skip it) and stores its sums
+        // in the slot of the first.
+        auto go = [&](auto nr_tag, auto f_tag) {
+            constexpr int NR = decltype(nr_tag)::value, F = decltype(f_tag)::value;
+            if (ks % F) return;
+            shrink_rows<DT, G, RMAX, KSC * F, NR, BIG>(p, rows, tok, r, proj, ks / F, ks, s_part);
+            __syncthreads();                                    // s_part is reused by the next record
+        };
+        using SF = SliceFactor<RMAX>;
+        if constexpr (RMAX >= 64) {
+            if (r > 32) { go(std::integral_constant<int, 16>{}, std::integral_constant<int, SF::F16>{}); continue; }
+        }
+        if constexpr (RMAX >= 32) {
+            if (r > 16) { go(std::integral_constant<int, 8>{}, std::integral_constant<int, SF::F8>{}); continue; }
+        }
+        if (r > 8) { go(std::integral_constant<int, 4>{}, std::integral_constant<int, SF::F4>{}); continue; }
+        go(std::integral_constant<int, 2>{}, std::integral_constant<int, SF::F2>{});
     }
-    if constexpr (RMAX >= 32) {
-        if (r > 16) { go(std::integral_constant<int, 8>{}, std::integral_constant<int, SF::F8>{}); return; }
-    }
-    if (r > 8) { go(std::integral_constant<int, 4>{}, std::integral_constant<int, SF::F4>{}); return; }
-    go(std::integral_constant<int, 2>{}, std::integral_constant<int, SF::F2>{});
 }
 
 template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
@@ -227,130 +234,135 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
     int proj = 0;
     while (proj + 1 < p.n_proj && id.q >= p.ex_end[proj]) proj++;
     const int cs = id.q - (proj ? p.ex_end[proj - 1] : 0);
-    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
-    int ntok = rec[0];
-    if (ntok <= 0) return;
-    ntok = ntok < G ? ntok : G;
     const int hout = p.hout[proj];
     const int ncc_out = hout >> 3;
     const int cc = cs * NTE + tid;
     const bool active = cc < ncc_out;
-    const int adapter = rec[1];
-    int r = rec[2];
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    const float scale = __builtin_bit_cast(float, rec[3]);
-    int tok[G];
-#pragma unroll
-    for (int k = 0; k < G; k++) {
-        const int t = k < ntok ? rec[4 + k] : -1;
-        tok[k] = (t >= 0 && t < p.T) ? t : -1;
-    }
-    const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
     uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y[proj]);
     const uint16_t *__restrict__ brows = static_cast<const uint16_t *>(p.b_rows[proj]);
+    const unsigned voff = (unsigned)(active ? cc : 0) * 16u;
+    const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
 
-    if (adapter < 0) {
-        if (!p.accumulate && active) {
+    // records id.b, id.b + stride, ... (see the shrink kernel)
+    for (int b = id.b; b < p.items_cap; b += p.rec_stride_ex) {
+        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+        int ntok = rec[0];
+        if (ntok <= 0) break;
+        ntok = ntok < G ? ntok : G;
+        const int adapter = rec[1];
+        int r = rec[2];
+        r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
+        const float scale = __builtin_bit_cast(float, rec[3]);
+        int tok[G];
+#pragma unroll
+        for (int k = 0; k < G; k++) {
+            const int t = k < ntok ? rec[4 + k] : -1;
+            tok[k] = (t >= 0 && t < p.T) ? t : -1;
+        }
+        const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+
+        if (adapter < 0) {
+            if (!p.accumulate && active) {
+#pragma unroll
+                for (int k = 0; k < G; k++)
+                    if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, zero16());
+            }
+            continue;
+        }
+
+        auto b_rows_of = [&](int j0, int (&out)[EB]) {              // rows of rank rows j0 .. j0+EB-1
+            if constexpr (EB % 4 == 0) {
+                const int4 *q = reinterpret_cast<const int4 *>(rows + j0);
+#pragma unroll
+                for (int m = 0; m < EB / 4; m++) {
+                    const int4 v = q[m];
+                    out[4 * m] = v.x; out[4 * m + 1] = v.y; out[4 * m + 2] = v.z; out[4 * m + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int jj = 0; jj < EB; jj++) out[jj] = rows[j0 + jj];
+            }
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++) out[jj] = (out[jj] >= 0 && out[jj] < pv.n_rows_b) ? out[jj] : -1;
+        };
+
+        // A rank row's address is the same for the whole workgroup (scalar registers) and a lane adds its column
+        // offset; an absent row reads row 0 and is zeroed afterwards, so a batch of loads is issued without a branch.
+        auto load_b = [&](int j0, uint4 (&out)[EB]) {
+            int br[EB];
+            b_rows_of(j0, br);
+            if constexpr (!BIG) {
+#pragma unroll
+                for (int jj = 0; jj < EB; jj++)
+                    out[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
+                return;
+            }
+#pragma unroll
+            for (int jj = 0; jj < EB; jj++) {
+                const int row = __builtin_amdgcn_readfirstlane(br[jj]);
+                const char *rp = reinterpret_cast<const char *>(brows) + (size_t)(row >= 0 ? row : 0) * (size_t)hout * 2u;
+                out[jj] = ldg16(rp + voff);
+                if (row < 0) out[jj] = zero16();
+            }
+        };
+        // Everything the first step needs is requested before the partial sums are fetched.
+        uint4 bv[EB];
+        uint4 yv[G];
+        if (active) {
+            load_b(0, bv);
 #pragma unroll
             for (int k = 0; k < G; k++)
-                if (tok[k] >= 0) stg16(y + (size_t)tok[k] * hout + (size_t)cc * 8, zero16());
+                yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
         }
-        return;
-    }
 
-    auto b_rows_of = [&](int j0, int (&out)[EB]) {              // rows of rank rows j0 .. j0+EB-1
-        if constexpr (EB % 4 == 0) {
-            const int4 *q = reinterpret_cast<const int4 *>(rows + j0);
+        // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
+        const int kstep = slice_factor<RMAX>(r);                   // the shrink filled every kstep-th slot
+        for (int e = tid; e < G * RMAX; e += NT) {
+            const int k = e / RMAX, j = e - k * RMAX;
+            float s = 0.f;
+            if (j < r && tok[k] >= 0) {
+                // eight slices' sums are requested at once (one round trip instead of one per slice) and added in
+                // ascending slice order
+                const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
+                for (int ks0 = 0; ks0 < n_ks; ks0 += 8 * kstep) {
+                    float t[8];
 #pragma unroll
-            for (int m = 0; m < EB / 4; m++) {
-                const int4 v = q[m];
-                out[4 * m] = v.x; out[4 * m + 1] = v.y; out[4 * m + 2] = v.z; out[4 * m + 3] = v.w;
-            }
-        } else {
+                    for (int u = 0; u < 8; u++) {
+                        const int ks = ks0 + u * kstep;
+                        t[u] = ks < n_ks ? src[(size_t)ks * RMAX] : 0.f;
+                    }
 #pragma unroll
-            for (int jj = 0; jj < EB; jj++) out[jj] = rows[j0 + jj];
-        }
-#pragma unroll
-        for (int jj = 0; jj < EB; jj++) out[jj] = (out[jj] >= 0 && out[jj] < pv.n_rows_b) ? out[jj] : -1;
-    };
-
-    // A rank row's address is the same for the whole workgroup (scalar registers) and a lane adds its column
-    // offset; an absent row reads row 0 and is zeroed afterwards, so a batch of loads is issued without a branch.
-    const unsigned voff = (unsigned)(active ? cc : 0) * 16u;
-    auto load_b = [&](int j0, uint4 (&out)[EB]) {
-        int br[EB];
-        b_rows_of(j0, br);
-        if constexpr (!BIG) {
-#pragma unroll
-            for (int jj = 0; jj < EB; jj++)
-                out[jj] = br[jj] >= 0 ? ldg16_stream(brows + (size_t)br[jj] * hout + (size_t)cc * 8) : zero16();
-            return;
-        }
-#pragma unroll
-        for (int jj = 0; jj < EB; jj++) {
-            const int row = __builtin_amdgcn_readfirstlane(br[jj]);
-            const char *rp = reinterpret_cast<const char *>(brows) + (size_t)(row >= 0 ? row : 0) * (size_t)hout * 2u;
-            out[jj] = ldg16(rp + voff);
-            if (row < 0) out[jj] = zero16();
-        }
-    };
-    // Everything the first step needs is requested before the partial sums are fetched.
-    uint4 bv[EB];
-    uint4 yv[G];
-    if (active) {
-        load_b(0, bv);
-#pragma unroll
-        for (int k = 0; k < G; k++)
-            yv[k] = (p.accumulate && tok[k] >= 0) ? ldg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8) : zero16();
-    }
-
-    // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
-    const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
-    const int kstep = slice_factor<RMAX>(r);                   // the shrink filled every kstep-th slot
-    for (int e = tid; e < G * RMAX; e += NT) {
-        const int k = e / RMAX, j = e - k * RMAX;
-        float s = 0.f;
-        if (j < r && tok[k] >= 0) {
-            // eight slices' sums are requested at once (one round trip instead of one per slice) and added in
-            // ascending slice order
-            const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
-            for (int ks0 = 0; ks0 < n_ks; ks0 += 8 * kstep) {
-                float t[8];
-#pragma unroll
-                for (int u = 0; u < 8; u++) {
-                    const int ks = ks0 + u * kstep;
-                    t[u] = ks < n_ks ? src[(size_t)ks * RMAX] : 0.f;
+                    for (int u = 0; u < 8; u++) s += t[u];
                 }
-#pragma unroll
-                for (int u = 0; u < 8; u++) s += t[u];
             }
+            s_v[k][j] = s * scale;
         }
-        s_v[k][j] = s * scale;
-    }
-    __syncthreads();
-    if (!active) return;
-
-    float o[G][8];
+        __syncthreads();
+        if (active) {
+            float o[G][8];
 #pragma unroll
-    for (int k = 0; k < G; k++) unpack8<DT>(yv[k], o[k]);
+            for (int k = 0; k < G; k++) unpack8<DT>(yv[k], o[k]);
 #pragma unroll 1
-    for (int j0 = 0; j0 < r; j0 += EB) {
-        if (j0 > 0) load_b(j0, bv);
+            for (int j0 = 0; j0 < r; j0 += EB) {
+                if (j0 > 0) load_b(j0, bv);
 #pragma unroll
-        for (int jj = 0; jj < EB; jj++) {
-            float f[8];
-            unpack8<DT>(bv[jj], f);
+                for (int jj = 0; jj < EB; jj++) {
+                    float f[8];
+                    unpack8<DT>(bv[jj], f);
 #pragma unroll
-            for (int k = 0; k < G; k++) {
-                const float vk = s_v[k][j0 + jj];
+                    for (int k = 0; k < G; k++) {
+                        const float vk = s_v[k][j0 + jj];
 #pragma unroll
-                for (int e = 0; e < 8; e++) o[k][e] = fmaf(vk, f[e], o[k][e]);
+                        for (int e = 0; e < 8; e++) o[k][e] = fmaf(vk, f[e], o[k][e]);
+                    }
+                }
             }
-        }
-    }
 #pragma unroll
-    for (int k = 0; k < G; k++)
-        if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
+            for (int k = 0; k < G; k++)
+                if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
+        }
+        __syncthreads();                                        // s_v is reused by the next record
+    }
 }
 
 // Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
@@ -393,119 +405,146 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
     int proj = 0;
     while (proj + 1 < p.n_proj && id.q >= p.ex_end[proj]) proj++;
     const int cs = id.q - (proj ? p.ex_end[proj - 1] : 0);
-    const int32_t *__restrict__ rec = p.work + (size_t)id.b * WORK_WORDS;
-    int ntok = rec[0];
-    if (ntok <= 0) return;
-    ntok = ntok < G ? ntok : G;
     const int hout = p.hout[proj];
-    const int adapter = rec[1];
-    int tok[G];
-#pragma unroll
-    for (int k = 0; k < G; k++) {
-        const int t = k < ntok ? rec[4 + k] : -1;
-        tok[k] = (t >= 0 && t < p.T) ? t : -1;
-    }
     uint16_t *__restrict__ y = static_cast<uint16_t *>(p.y[proj]);
     const int col_begin = cs * SLICE;
     const int col_end = col_begin + SLICE < hout ? col_begin + SLICE : hout;
     // y rows are handled by the first G * 32 threads: thread t -> token t / 32, 8 columns from (t % 32) * 8 of the sub-tile
     const int yk = tid >> 5, yc = (tid & 31) * 8;
-    int ytok = -1;
-#pragma unroll
-    for (int k = 0; k < G; k++) ytok = yk == k ? tok[k] : ytok;
-
-    if (adapter < 0 || adapter >= p.pool.n_adapters) {
-        if (!p.accumulate && ytok >= 0)
-            for (int c0 = col_begin; c0 < col_end; c0 += SUB)
-                if (c0 + yc < col_end) stg16(y + (size_t)ytok * hout + c0 + yc, zero16());
-        return;
-    }
-    const float scale = __builtin_bit_cast(float, rec[3]) * p.pool.uniform_scale;
-    const uint16_t *__restrict__ bt = static_cast<const uint16_t *>(p.b_rows[proj]) +
-                                      (size_t)adapter * (size_t)p.ref_layers * (size_t)hout * R;
     const int part = tid % LPC;                                 // which 8 ranks of a column this lane multiplies
-
-    uint4 bv[LPC], bn[LPC];
-    auto load_sub = [&](int c0, uint4 (&out)[LPC]) {
-        // chunk 256 i + t of the sub-tile's run: column c0 + i * CPP + t / LPC, ranks part * 8 ..
-#pragma unroll
-        for (int i = 0; i < LPC; i++) {
-            const int col = c0 + i * CPP + tid / LPC;
-            out[i] = col < col_end ? ldg16_stream(bt + (size_t)c0 * R + ((size_t)i * 256 + tid) * 8) : zero16();
-        }
-    };
-    load_sub(col_begin, bv);
-    uint4 yv = zero16();
-    if (p.accumulate && ytok >= 0 && col_begin + yc < col_end) yv = ldg16_stream(y + (size_t)ytok * hout + col_begin + yc);
-
-    // v = scaling * (sum of the slices' partial sums), slices added in ascending order
     const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
-    for (int e = tid; e < G * RMAX; e += 256) {
-        const int k = e / RMAX, j = e - k * RMAX;
-        float s = 0.f;
-        if (j < R && tok[k] >= 0) {
-            const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
-            for (int ks0 = 0; ks0 < n_ks; ks0 += 8) {
-                float t8[8];
-#pragma unroll
-                for (int u = 0; u < 8; u++) t8[u] = ks0 + u < n_ks ? src[(size_t)(ks0 + u) * RMAX] : 0.f;
-#pragma unroll
-                for (int u = 0; u < 8; u++) s += t8[u];
-            }
-        }
-        s_v[k][j] = s * scale;
-    }
-    __syncthreads();
-    float vr[G][8];                                             // this lane's 8 intermediates of every token
-#pragma unroll
-    for (int k = 0; k < G; k++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) vr[k][e] = s_v[k][part * 8 + e];
 
-    int buf = 0;
-#pragma unroll 1
-    for (int c0 = col_begin; c0 < col_end; c0 += SUB, buf ^= 1) {
-        const bool more = c0 + SUB < col_end;
-        if (more) load_sub(c0 + SUB, bn);
-        uint4 yn = zero16();
-        if (more && p.accumulate && ytok >= 0 && c0 + SUB + yc < col_end) yn = ldg16_stream(y + (size_t)ytok * hout + c0 + SUB + yc);
+    // records id.b, id.b + stride, ... (see the shrink kernel)
+    for (int b = id.b; b < p.items_cap; b += p.rec_stride_ex) {
+        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+        int ntok = rec[0];
+        if (ntok <= 0) break;
+        ntok = ntok < G ? ntok : G;
+        const int adapter = rec[1];
+        int tok[G];
 #pragma unroll
-        for (int i = 0; i < LPC; i++) {
-            float f[8];
-            unpack8<DT>(bv[i], f);
+        for (int k = 0; k < G; k++) {
+            const int t = k < ntok ? rec[4 + k] : -1;
+            tok[k] = (t >= 0 && t < p.T) ? t : -1;
+        }
+        int ytok = -1;
 #pragma unroll
-            for (int k = 0; k < G; k++) {
-                float d = 0.f;
+        for (int k = 0; k < G; k++) ytok = yk == k ? tok[k] : ytok;
+
+        if (adapter < 0 || adapter >= p.pool.n_adapters) {
+            if (!p.accumulate && ytok >= 0)
+                for (int c0 = col_begin; c0 < col_end; c0 += SUB)
+                    if (c0 + yc < col_end) stg16(y + (size_t)ytok * hout + c0 + yc, zero16());
+            continue;
+        }
+        const float scale = __builtin_bit_cast(float, rec[3]) * p.pool.uniform_scale;
+        const uint16_t *__restrict__ bt = static_cast<const uint16_t *>(p.b_rows[proj]) +
+                                          (size_t)adapter * (size_t)p.ref_layers * (size_t)hout * R;
+
+        uint4 bv[LPC], bn[LPC];
+        auto load_sub = [&](int c0, uint4 (&out)[LPC]) {
+            // chunk 256 i + t of the sub-tile's run: column c0 + i * CPP + t / LPC, ranks part * 8 ..
 #pragma unroll
-                for (int e = 0; e < 8; e++) d = fmaf(vr[k][e], f[e], d);
-                d = group_sum<LPC>(d);
-                if (part == 0) s_out[buf][k][i * CPP + tid / LPC] = d;
+            for (int i = 0; i < LPC; i++) {
+                const int col = c0 + i * CPP + tid / LPC;
+                out[i] = col < col_end ? ldg16_stream(bt + (size_t)c0 * R + ((size_t)i * 256 + tid) * 8) : zero16();
             }
-        }
-        __syncthreads();                                        // also orders this buffer's reads of two steps ago before these writes
-        if (ytok >= 0 && c0 + yc < col_end) {
-            float o[8];
-            unpack8<DT>(yv, o);                                 // zeros when not accumulating
-            const float4_t d0 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc]);
-            const float4_t d1 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc + 4]);
-            o[0] += d0[0]; o[1] += d0[1]; o[2] += d0[2]; o[3] += d0[3];
-            o[4] += d1[0]; o[5] += d1[1]; o[6] += d1[2]; o[7] += d1[3];
-            stg16_stream(y + (size_t)ytok * hout + c0 + yc, pack8<DT>(o));
-        }
+        };
+        load_sub(col_begin, bv);
+        uint4 yv = zero16();
+        if (p.accumulate && ytok >= 0 && col_begin + yc < col_end) yv = ldg16_stream(y + (size_t)ytok * hout + col_begin + yc);
+
+        // v = scaling * (sum of the slices' partial sums), slices added in ascending order
+        for (int e = tid; e < G * RMAX; e += 256) {
+            const int k = e / RMAX, j = e - k * RMAX;
+            float s = 0.f;
+            if (j < R && tok[k] >= 0) {
+                const float *src = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max) * RMAX + j;
+                for (int ks0 = 0; ks0 < n_ks; ks0 += 8) {
+                    float t8[8];
 #pragma unroll
-        for (int i = 0; i < LPC; i++) bv[i] = bn[i];
-        yv = yn;
+                    for (int u = 0; u < 8; u++) t8[u] = ks0 + u < n_ks ? src[(size_t)(ks0 + u) * RMAX] : 0.f;
+#pragma unroll
+                    for (int u = 0; u < 8; u++) s += t8[u];
+                }
+            }
+            s_v[k][j] = s * scale;
+        }
+        __syncthreads();
+        float vr[G][8];                                             // this lane's 8 intermediates of every token
+#pragma unroll
+        for (int k = 0; k < G; k++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) vr[k][e] = s_v[k][part * 8 + e];
+
+        int buf = 0;
+#pragma unroll 1
+        for (int c0 = col_begin; c0 < col_end; c0 += SUB, buf ^= 1) {
+            const bool more = c0 + SUB < col_end;
+            if (more) load_sub(c0 + SUB, bn);
+            uint4 yn = zero16();
+            if (more && p.accumulate && ytok >= 0 && c0 + SUB + yc < col_end) yn = ldg16_stream(y + (size_t)ytok * hout + c0 + SUB + yc);
+#pragma unroll
+            for (int i = 0; i < LPC; i++) {
+                float f[8];
+                unpack8<DT>(bv[i], f);
+#pragma unroll
+                for (int k = 0; k < G; k++) {
+                    float d = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) d = fmaf(vr[k][e], f[e], d);
+                    d = group_sum<LPC>(d);
+                    if (part == 0) s_out[buf][k][i * CPP + tid / LPC] = d;
+                }
+            }
+            __syncthreads();                                        // also orders this buffer's reads of two steps ago before these writes
+            if (ytok >= 0 && c0 + yc < col_end) {
+                float o[8];
+                unpack8<DT>(yv, o);                                 // zeros when not accumulating
+                const float4_t d0 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc]);
+                const float4_t d1 = *reinterpret_cast<const float4_t *>(&s_out[buf][yk][yc + 4]);
+                o[0] += d0[0]; o[1] += d0[1]; o[2] += d0[2]; o[3] += d0[3];
+                o[4] += d1[0]; o[5] += d1[1]; o[6] += d1[2]; o[7] += d1[3];
+                stg16_stream(y + (size_t)ytok * hout + c0 + yc, pack8<DT>(o));
+            }
+#pragma unroll
+            for (int i = 0; i < LPC; i++) bv[i] = bn[i];
+            yv = yn;
+        }
+        __syncthreads();                                        // s_v and s_out are reused by the next record
     }
 }
 
-template <int DT, int G, int R>
-static int launch_pair_bt(const BgmvArgs &a, hipStream_t s)
+// Records a launch covers (a multiple of 8, one per XCD residue): every workgroup walks records b, b + stride, ...
+// The host only knows an upper bound on the records in use (items_cap: T/G full pieces plus one short piece per
+// adapter present); a grid over the whole bound spends about a nanosecond per workgroup of an empty record on
+// dispatch alone, which is a tenth of a launch of thousands of slices.  The stride is never below ceil(T/G)
+// (that many records are in use whenever every token has an adapter entry) and large enough for the launch to
+// hold a few rounds of workgroups, so that small batches keep one workgroup per record.
+#ifndef MLORA_GRID_TARGET
+#define MLORA_GRID_TARGET 3072
+#endif
+template <int G>
+static int record_stride(const BgmvArgs &a, int slices)
 {
+    long long want = (a.T + G - 1) / G;
+    const long long fill = (MLORA_GRID_TARGET + slices - 1) / slices;
+    want = want > fill ? want : fill;
+    want = (want + 7) / 8 * 8;
+    return want < a.items_cap ? (int)want : a.items_cap;
+}
+
+template <int DT, int G, int R>
+static int launch_pair_bt(const BgmvArgs &a0, hipStream_t s)
+{
+    BgmvArgs a = a0;
+    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1]);
+    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1]);
     constexpr int RMAX = R <= 16 ? 16 : (R <= 32 ? 32 : 64);
     constexpr int KSC = Slices<RMAX>::KSC;
     static_assert(Slices<RMAX>::NTE * 8 == 2048, "the transposed-B expand walks 2048-column slices");
-    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.items_cap;
-    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.items_cap;
+    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.rec_stride_sh;
+    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.rec_stride_ex;
     if (n_sh <= 0 || n_ex <= 0) return 0;
     if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC, false>), dim3((unsigned)n_sh), dim3(256), 0, s, a);
@@ -539,10 +578,13 @@ static int launch_bt_dt(const BgmvArgs &a, int group, int r, hipStream_t s)
 }
 
 template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
-static int launch_pair(const BgmvArgs &a, hipStream_t s)
+static int launch_pair(const BgmvArgs &a0, hipStream_t s)
 {
-    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.items_cap;
-    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.items_cap;
+    BgmvArgs a = a0;
+    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1]);
+    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1]);
+    const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.rec_stride_sh;
+    const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.rec_stride_ex;
     if (n_sh <= 0 || n_ex <= 0) return 0;
     if (n_sh > 0x7fffffffLL || n_ex > 0x7fffffffLL) return (int)hipErrorInvalidValue;
     hipLaunchKernelGGL((bgmv_shrink_kernel<DT, G, RMAX, KSC, BIG>), dim3((unsigned)n_sh), dim3(256), 0, s, a);

@@ -218,8 +218,12 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
         const_cast<uint16_t *>(wgt), (short)0, (int)((size_t)hin * hout * 2), 0x00020000);
     // The loads are written as inline assembly: the compiler's own bookkeeping of loads that land in LDS waits
     // for all of them before any LDS read that follows, which would serialise the ring; here the waits are
-    // explicit (GL_WAIT_LOADS below).  M0 carries the LDS address of the wavefront's 1 KiB chunk; nothing else
-    // in this kernel uses M0.
+    // explicit (GL_WAIT_LOADS below).  M0 carries the LDS address of the wavefront's 1 KiB chunk.  The compiler
+    // keeps M0 as a reserved register: it rejects "m0" in a clobber list ("clobber list contains reserved
+    // registers") and writes M0 itself right before each of its own uses; nothing in this kernel makes it
+    // emit one (no LDS-bound load builtin, no relative register move, no message with an M0 payload), and the
+    // build-time resource check fails if the kernel's code ever reads M0 outside these statements.  The
+    // "memory" clobber keeps LDS and global accesses from being moved across a load.
     typedef int gl_i32x4 __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) unsigned char lds_byte;
     auto rsrc_words = [](const void *base, size_t bytes) {
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(G_NT, 1) void gemm_lora_kernel(const GemmLoraArgs p
     const gl_i32x4 wrw = rsrc_words(wgt, (size_t)hin * hout * 2);
     auto dma1 = [](const gl_i32x4 &rs, unsigned lds_addr, unsigned voff, unsigned soff) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                     :: "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff));
+                     :: "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff) : "memory");
     };
     // the 8 loads of one K step: 4 of x, 4 of W
     auto dma = [&](unsigned char *stage, int ks) {

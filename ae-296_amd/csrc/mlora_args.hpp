@@ -59,6 +59,9 @@ struct BgmvArgs {
     // the number of shrink / expand slices of projections 0..p
     int sh_end[MAX_PROJ];
     int ex_end[MAX_PROJ];
+    // two-launch form: records the shrink / expand grid covers; a workgroup walks records b, b + stride, ... < items_cap
+    // (set by the launcher)
+    int rec_stride_sh, rec_stride_ex;
 };
 
 constexpr int SCATTER_MAX_JOBS = 16;
