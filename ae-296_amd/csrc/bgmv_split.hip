@@ -23,14 +23,27 @@
 namespace mlora {
 
 
-// How a launch treats the adapter rows, chosen by the host from the size of the batch:
-//   BIG = false: a hot adapter's work items all run at once (the launch is about one round of workgroups), rows
-//     pass through L2 once and are read with the nontemporal hint so that they do not displace records and sums;
-//   BIG = true: the launch is many rounds of workgroups, the items of a hot adapter follow each other on one XCD
-//     and find its rows in L2 only if they are kept: ordinary loads, and the expand keeps fewer rows in flight per
-//     lane (more resident wavefronts instead), which measured faster at that size.
+// How a launch reads the adapter rows, chosen by the host from the size of the batch:
+//   HOT = false: the launch is about one round of workgroups, all items of an adapter run at the same time and the
+//     rows pass through L2 once: nontemporal loads, which do not displace records and sums;
+//   HOT = true: a launch of many rounds of workgroups; the items of a much-used adapter follow each other on one
+//     XCD and find its rows in L2 only if they are kept: ordinary loads.  (Choosing per item, by whether the
+//     neighbouring records name the same adapter, measured slower than either.)
+template <bool HOT>
+__device__ __forceinline__ uint4 ld_rows(const void *p) { if constexpr (HOT) return ldg16(p); else return ldg16_stream(p); }
+
+// A work record as the kernels read it.  In a one-round launch (no loop over records) an ordinary pointer: the
+// compiler already fetches the header with scalar loads and the allocation it reaches with that is the measured
+// best; in a launch of many rounds the record is read as constant memory, which keeps the header loads scalar
+// inside the loop over records.
+template <bool BIG> struct RecPtr { typedef const int32_t *__restrict__ type; };
+template <> struct RecPtr<true> { typedef const_i32_ptr type; };
 template <bool BIG>
-__device__ __forceinline__ uint4 ld_rows(const void *p) { if constexpr (BIG) return ldg16(p); else return ldg16_stream(p); }
+__device__ __forceinline__ typename RecPtr<BIG>::type record_at(const int32_t *work, int b)
+{
+    if constexpr (BIG) return as_const(work + (size_t)b * WORK_WORDS);
+    else return work + (size_t)b * WORK_WORDS;
+}
 
 struct ItemId { int b, q; };
 
@@ -46,22 +59,25 @@ __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
 // Slices of the launch's width (Slices<RMAX>::KSC) that one shrink workgroup takes, by the rank bucket of
 // its item (more than 32, 17..32, 9..16, at most 8 rank rows): the bytes of a workgroup grow with
 // rank x width, so an item of low rank in a launch sized for rank 64 takes wider slices.
-template <int RMAX> struct SliceFactor;
-template <> struct SliceFactor<16> { static constexpr int F16 = 1, F8 = 1, F4 = 1, F2 = 1; };
-template <> struct SliceFactor<32> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
-template <> struct SliceFactor<64> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
-template <int RMAX>
+#ifndef MLORA_F8BIG
+#define MLORA_F8BIG 2
+#endif
+template <int RMAX, bool BIG> struct SliceFactor;
+template <bool BIG> struct SliceFactor<16, BIG> { static constexpr int F16 = 1, F8 = 1, F4 = 1, F2 = 1; };
+template <bool BIG> struct SliceFactor<32, BIG> { static constexpr int F16 = 1, F8 = BIG ? MLORA_F8BIG : 1, F4 = 2, F2 = 4; };
+template <bool BIG> struct SliceFactor<64, BIG> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
+template <int RMAX, bool BIG>
 __device__ __forceinline__ int slice_factor(int r)
 {
-    using SF = SliceFactor<RMAX>;
+    using SF = SliceFactor<RMAX, BIG>;
     return r > 32 ? SF::F16 : (r > 16 ? SF::F8 : (r > 8 ? SF::F4 : SF::F2));
 }
 
 // Shrink of one (item, projection, column slice) over the first 4 * NR rank rows (NR per 16-lane
 // row).  The caller picks the smallest NR that covers the item's rank, so an adapter of rank 8 in a
 // pool that goes up to rank 64 issues loads for 8 rows, not 64.
-template <int DT, int G, int RMAX, int KSC, int NR, bool BIG>
-__device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__restrict__ rows, const int (&tok)[G],
+template <int DT, int G, int RMAX, int KSC, int NR, bool HOT, class RowsPtr>
+__device__ __forceinline__ void shrink_rows(const BgmvArgs &p, RowsPtr rows, const int (&tok)[G],
                                             int r, int proj, int ks, int slot, float (&s_part)[4][G][RMAX])
 {
     constexpr int NW = 4;
@@ -114,7 +130,7 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
 #pragma unroll
                 for (int k = 0; k < G; k++) xv[k][u] = ldg16_stream(xp[k] + (it0 + u) * 16);
 #pragma unroll
-                for (int i = 0; i < NR; i++) av[i][u] = ld_rows<BIG>(ap[i] + (it0 + u) * 16);
+                for (int i = 0; i < NR; i++) av[i][u] = ld_rows<HOT>(ap[i] + (it0 + u) * 16);
             }
 #pragma unroll
             for (int u = 0; u < U; u++)
@@ -134,7 +150,7 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, const int32_t *__
 #pragma unroll
             for (int k = 0; k < G; k++) xv[k] = ldg16_stream(xp[k] + cs);
 #pragma unroll
-            for (int i = 0; i < NR; i++) av[i] = ld_rows<BIG>(ap[i] + cs);
+            for (int i = 0; i < NR; i++) av[i] = ld_rows<HOT>(ap[i] + cs);
 #pragma unroll
             for (int k = 0; k < G; k++) {
                 xv[k].x = cv ? xv[k].x : 0u; xv[k].y = cv ? xv[k].y : 0u;
@@ -181,8 +197,9 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
     // host's upper bound on them (the records in use of one XCD residue are a prefix, so the first empty one ends
     // the walk).  Most batches need one pass; what a grid over the whole bound would spend on dispatching
     // workgroups of empty records is saved.
-    for (int b = id.b; b < p.items_cap; b += p.rec_stride_sh) {
-        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+    int b = id.b;
+    do {
+        const typename RecPtr<BIG>::type rec = record_at<BIG>(p.work, b);
         int ntok = rec[0];
         if (ntok <= 0) break;
         ntok = ntok < G ? ntok : G;
@@ -196,7 +213,7 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
             const int t = k < ntok ? rec[4 + k] : -1;
             tok[k] = (t >= 0 && t < p.T) ? t : -1;
         }
-        const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+        const typename RecPtr<BIG>::type rows = rec + WORK_ROWS_AT;
 
         // r is uniform over the workgroup: a scalar branch, no divergence.  An item of a lower rank bucket
         // takes F consecutive slices in one workgroup (the others of the F skip it) and stores its sums
@@ -205,9 +222,9 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
             constexpr int NR = decltype(nr_tag)::value, F = decltype(f_tag)::value;
             if (ks % F) return;
             shrink_rows<DT, G, RMAX, KSC * F, NR, BIG>(p, rows, tok, r, proj, ks / F, ks, s_part);
-            __syncthreads();                                    // s_part is reused by the next record
+            if constexpr (BIG) __syncthreads();                 // s_part is reused by the next record
         };
-        using SF = SliceFactor<RMAX>;
+        using SF = SliceFactor<RMAX, BIG>;
         if constexpr (RMAX >= 64) {
             if (r > 32) { go(std::integral_constant<int, 16>{}, std::integral_constant<int, SF::F16>{}); continue; }
         }
@@ -216,14 +233,17 @@ __global__ __launch_bounds__(256) void bgmv_shrink_kernel(const BgmvArgs p)
         }
         if (r > 8) { go(std::integral_constant<int, 4>{}, std::integral_constant<int, SF::F4>{}); continue; }
         go(std::integral_constant<int, 2>{}, std::integral_constant<int, SF::F2>{});
-    }
+    } while (BIG && (b += p.rec_stride_sh) < p.items_cap);
 }
 
 template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 {
     constexpr int NT = NTE;                                    // one 16-byte chunk of the slice per thread
-    constexpr int EBW = BIG ? 4 : 8;
+#ifndef MLORA_EBW_BIG
+#define MLORA_EBW_BIG 8
+#endif
+    constexpr int EBW = BIG ? MLORA_EBW_BIG : 8;
     constexpr int EB = RMAX < EBW ? RMAX : EBW;                 // B rank rows in flight per lane
     __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
 
@@ -244,8 +264,9 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
     const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
 
     // records id.b, id.b + stride, ... (see the shrink kernel)
-    for (int b = id.b; b < p.items_cap; b += p.rec_stride_ex) {
-        const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
+    int b = id.b;
+    do {
+        const typename RecPtr<BIG>::type rec = record_at<BIG>(p.work, b);
         int ntok = rec[0];
         if (ntok <= 0) break;
         ntok = ntok < G ? ntok : G;
@@ -259,7 +280,7 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
             const int t = k < ntok ? rec[4 + k] : -1;
             tok[k] = (t >= 0 && t < p.T) ? t : -1;
         }
-        const int32_t *__restrict__ rows = rec + WORK_ROWS_AT;
+        const typename RecPtr<BIG>::type rows = rec + WORK_ROWS_AT;
 
         if (adapter < 0) {
             if (!p.accumulate && active) {
@@ -271,7 +292,7 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         }
 
         auto b_rows_of = [&](int j0, int (&out)[EB]) {              // rows of rank rows j0 .. j0+EB-1
-            if constexpr (EB % 4 == 0) {
+            if constexpr (!BIG && EB % 4 == 0) {
                 const int4 *q = reinterpret_cast<const int4 *>(rows + j0);
 #pragma unroll
                 for (int m = 0; m < EB / 4; m++) {
@@ -316,7 +337,7 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
         }
 
         // v = scaling * (sum of the slices' partial sums), slices added in ascending order.
-        const int kstep = slice_factor<RMAX>(r);                   // the shrink filled every kstep-th slot
+        const int kstep = slice_factor<RMAX, BIG>(r);                   // the shrink filled every kstep-th slot
         for (int e = tid; e < G * RMAX; e += NT) {
             const int k = e / RMAX, j = e - k * RMAX;
             float s = 0.f;
@@ -361,8 +382,8 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
             for (int k = 0; k < G; k++)
                 if (tok[k] >= 0) stg16_stream(y + (size_t)tok[k] * hout + (size_t)cc * 8, pack8<DT>(o[k]));
         }
-        __syncthreads();                                        // s_v is reused by the next record
-    }
+        if constexpr (BIG) __syncthreads();                     // s_v is reused by the next record
+    } while (BIG && (b += p.rec_stride_ex) < p.items_cap);
 }
 
 // Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
@@ -370,7 +391,10 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 // on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
 template <int RMAX> struct Slices;
 template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
-template <> struct Slices<32> { static constexpr int KSC = 128, NTE = 256; };
+#ifndef MLORA_KSC32
+#define MLORA_KSC32 128
+#endif
+template <> struct Slices<32> { static constexpr int KSC = MLORA_KSC32, NTE = 256; };
 template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
 // Sum over each aligned group of LPC lanes (1, 2, 4 or 8); every lane of the group gets the sum.
 template <int LPC>
@@ -414,8 +438,8 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
     const int part = tid % LPC;                                 // which 8 ranks of a column this lane multiplies
     const int n_ks = ((p.hin[proj] >> 3) + KSC - 1) / KSC;
 
-    // records id.b, id.b + stride, ... (see the shrink kernel)
-    for (int b = id.b; b < p.items_cap; b += p.rec_stride_ex) {
+    const int b = id.b;
+    do {
         const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
         int ntok = rec[0];
         if (ntok <= 0) break;
@@ -511,8 +535,7 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
             for (int i = 0; i < LPC; i++) bv[i] = bn[i];
             yv = yn;
         }
-        __syncthreads();                                        // s_v and s_out are reused by the next record
-    }
+    } while (false);
 }
 
 // Records a launch covers (a multiple of 8, one per XCD residue): every workgroup walks records b, b + stride, ...
@@ -525,8 +548,9 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
 #define MLORA_GRID_TARGET 3072
 #endif
 template <int G>
-static int record_stride(const BgmvArgs &a, int slices)
+static int record_stride(const BgmvArgs &a, int slices, bool big)
 {
+    if (!big) return a.items_cap;                               // about one round of workgroups: one per record
     long long want = (a.T + G - 1) / G;
     const long long fill = (MLORA_GRID_TARGET + slices - 1) / slices;
     want = want > fill ? want : fill;
@@ -538,8 +562,8 @@ template <int DT, int G, int R>
 static int launch_pair_bt(const BgmvArgs &a0, hipStream_t s)
 {
     BgmvArgs a = a0;
-    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1]);
-    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1]);
+    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1], false);
+    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1], false);
     constexpr int RMAX = R <= 16 ? 16 : (R <= 32 ? 32 : 64);
     constexpr int KSC = Slices<RMAX>::KSC;
     static_assert(Slices<RMAX>::NTE * 8 == 2048, "the transposed-B expand walks 2048-column slices");
@@ -581,8 +605,8 @@ template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 static int launch_pair(const BgmvArgs &a0, hipStream_t s)
 {
     BgmvArgs a = a0;
-    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1]);
-    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1]);
+    a.rec_stride_sh = record_stride<G>(a, a.sh_end[a.n_proj - 1], BIG);
+    a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1], BIG);
     const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.rec_stride_sh;
     const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.rec_stride_ex;
     if (n_sh <= 0 || n_ex <= 0) return 0;

@@ -20,6 +20,18 @@ __device__ __forceinline__ uint4 ldg16(const void *p) { return *reinterpret_cast
 __device__ __forceinline__ void stg16(void *p, uint4 v) { *reinterpret_cast<uint4 *>(p) = v; }
 __device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 
+// The same address seen as constant memory (address space 4): data that no launch of the running kernel writes
+// (work records, tile records and sums written by an earlier launch).  A load through such a pointer whose address
+// is uniform over the wavefront is a scalar load into SGPRs; through an ordinary global pointer the compiler only
+// does that while it can prove that no store of the kernel comes before the load, which a loop over work items
+// with a store at its end rules out.
+template <class T>
+__device__ __forceinline__ const __attribute__((address_space(4))) T *as_const(const T *p)
+{
+    return (const __attribute__((address_space(4))) T *)(__UINTPTR_TYPE__)p;
+}
+typedef const __attribute__((address_space(4))) int32_t *const_i32_ptr;
+
 // Streaming forms for data that is read or written once per launch (adapter rows, activations,
 // outputs): the nontemporal hint keeps these lines from displacing the small data every workgroup
 // re-reads (work records, partial sums) and measurably shortens the launches.
