@@ -562,7 +562,10 @@ SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
     // shrink workgroups: about three per CU for a single projection; a call over several projections
     // has that many already with fewer splits, and fewer splits mean less partial-sum traffic
     const long long per_split = (long long)w.max_tiles * n_proj;
-    const long long target = n_proj > 1 ? 2048 : 768;
+#ifndef MLORA_SG_TARGET
+#define MLORA_SG_TARGET 2048
+#endif
+    const long long target = n_proj > 1 ? MLORA_SG_TARGET : 768;
     long long ks = (target + per_split - 1) / per_split;
     w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : (int)ks);
     // a projection with a longer K than the others of its call gets proportionally more splits (up to three
@@ -603,7 +606,10 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
         int ks = (int)(((long long)w.ksplit * a.pr[p].hin + hin_min / 2) / (hin_min > 0 ? hin_min : 1));
         a.pr[p].ksplit = ks < w.ksplit ? w.ksplit : (ks > w.ks_cap ? w.ks_cap : ks);
         // 512 columns per expand workgroup amortise the V operand; fewer when that leaves the chip idle
-        int cols = 512;
+#ifndef MLORA_SG_COLS
+#define MLORA_SG_COLS 512
+#endif
+        int cols = MLORA_SG_COLS;
         if (a.n_proj == 1)
             while (cols > 128 && (long long)w.max_tiles * ((a.pr[p].hout + cols - 1) / cols) < 1024) cols >>= 1;
         a.pr[p].cols = cols;

@@ -127,6 +127,34 @@ def plan_decode(tok_adapter: torch.Tensor, pool: AdapterPool, group: Optional[in
     return out
 
 
+# ---------------------------------------------------------------------- two halves of a mixed batch side by side
+class SideStream:
+    """A second stream (default priority) with its fork and join events.  The decode tokens and the prefill
+    segments of a mixed batch touch different rows of x and y and only read the pool, so their launches need no
+    order between them: `side_by_side` puts one half on this stream and joins before it returns, and each half's
+    short tail of workgroups overlaps the other half's launches.  Works eagerly and under HIP graph capture (the
+    fork and the join become graph edges)."""
+
+    def __init__(self, device=None):
+        self.stream = torch.cuda.Stream(device=device)
+        self.fork = torch.cuda.Event()
+        self.join = torch.cuda.Event()
+
+
+def side_by_side(side: SideStream, on_side, on_main) -> None:
+    """Run `on_side()` on the side stream and `on_main()` on the current stream, both after everything already
+    queued on the current stream; what follows on the current stream waits for both.  The two callables must
+    not share a plan's intermediate buffers (a decode plan and a prefill plan never do)."""
+    main = torch.cuda.current_stream()
+    side.fork.record(main)
+    side.stream.wait_event(side.fork)
+    with torch.cuda.stream(side.stream):
+        on_side()
+    on_main()
+    side.join.record(side.stream)
+    main.wait_event(side.join)
+
+
 # ---------------------------------------------------------------------- decode
 def bgmv(ys: Sequence[torch.Tensor], xs: Sequence[torch.Tensor], pool: AdapterPool, layer: int,
          projs: Sequence[str], tok_adapter: torch.Tensor, plan: Optional[DecodePlan] = None,

@@ -745,6 +745,8 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
         pre = dict(ss=ss, sl=sl, sa=sa, T=Tp, x=px, y=py, ws=mlora.sgmv_workspace(Tp, n_seg, dev, n_proj=len(projs)),
                    adapters=seg_adapter)
 
+    side = mlora.SideStream(dev) if (pre is not None and not args.one_stream) else None
+
     def bgmv_layers():
         for l in range(L):
             mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
@@ -757,8 +759,18 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
             return
         pplan = mlora.plan_prefill(pre["ss"], pre["sl"], pre["sa"], pre["T"], pool, workspace=pre["ws"])
         for l in range(L):
-            mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
-            mlora.sgmv_multi([pre["y"][p] for p in projs], [pre["x"][_IN[p]] for p in projs], pool, l, projs, pplan)
+            def decode_half(l=l):
+                mlora.bgmv(ys[l], [xs[l][_IN[p]] for p in projs], pool, l, projs, tok, plan=plan, fused=fused)
+
+            def prefill_half(l=l):
+                mlora.sgmv_multi([pre["y"][p] for p in projs], [pre["x"][_IN[p]] for p in projs], pool, l, projs, pplan)
+
+            if side is None:
+                decode_half()
+                prefill_half()
+            else:
+                # the two halves of a layer run side by side and are joined before the next layer starts
+                mlora.side_by_side(side, prefill_half, decode_half)
 
     step()
     torch.cuda.synchronize()
@@ -843,6 +855,8 @@ def main():
     ap.add_argument("--split", action="store_true", help="decode: force the shrink + expand pair also where the host layer would pick the fused launch")
     ap.add_argument("--fused", action="store_true", help="decode: one fused launch per layer instead of the shrink + expand pair; c4: one SGMV call per projection "
                          "instead of one call over the seven")
+    ap.add_argument("--one-stream", action="store_true", help="c5: decode and prefill launches of a layer one after the other on one stream "
+                                                              "instead of side by side on two")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--eager", action="store_true", help="decode: also time the step launched eagerly (config.eager_ms_per_step)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
