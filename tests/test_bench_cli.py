@@ -30,3 +30,24 @@ def test_algorithmic_bytes_formula():
     assert set(bench.DECODE) >= {"c1", "c2", "c3", "c5", "maf128", "maf256", "maf512"}
     for name, cfg in bench.DECODE.items():
         assert cfg["T"] > 0 and cfg["layers"] > 0 and all(p in bench._IN for p in cfg["projs"]), name
+
+
+def test_traffic_figures_come_from_the_tracked_profiles():
+    """`roofline.traffic` is not a constant in bench.py: it is the `hbm_bytes_...` line of the workload's summary
+    under profiles/, which also states the counter commands and scale factors it came from."""
+    import re
+    sys.path.insert(0, ROOT)
+    import bench
+    for workload, (path, key) in bench.TRAFFIC_SOURCE.items():
+        text = open(os.path.join(ROOT, path)).read()
+        m = re.search(r"^\s*%s:\s*(\d+)\s*$" % re.escape(key), text, re.M)
+        assert m, f"{path} has no `{key}:` line"
+        value, source = bench.traffic_of(workload)
+        assert value == float(m.group(1)) and path in source
+        assert "rocprofv3 --pmc FETCH_SIZE" in text and "rocprofv3 --pmc WRITE_SIZE" in text and "FETCH_SIZE x" in text
+        assert f"bench.py --workload {workload}" in text
+    # every summary names the full command that produced it and runs committed files only
+    for name in os.listdir(os.path.join(ROOT, "profiles")):
+        text = open(os.path.join(ROOT, "profiles", name)).read()
+        assert "command: rocprofv3 --kernel-trace --stats" in text and "python3 bench.py" in text, name
+        assert "_work" not in text, name
