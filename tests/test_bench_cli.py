@@ -50,4 +50,4 @@ def test_traffic_figures_come_from_the_tracked_profiles():
     for name in os.listdir(os.path.join(ROOT, "profiles")):
         text = open(os.path.join(ROOT, "profiles", name)).read()
         assert "command: rocprofv3 --kernel-trace --stats" in text and "python3 bench.py" in text, name
-        assert "_work" not in text, name
+        assert "_work/" not in text, name
