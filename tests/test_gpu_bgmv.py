@@ -349,3 +349,31 @@ def test_bgmv_config5_one_layer_full_pool():
     torch.cuda.synchronize()
     for p in names:
         assert torch.allclose(ys[p].float(), want[p][o], rtol=RTOL, atol=ATOL), p
+
+
+@pytest.mark.parametrize("group", [4, 2])
+def test_bgmv_many_round_launch_walks_several_records(group):
+    """A launch of many rounds of workgroups (here 8 shrink slices x 1700 possible records) covers fewer records
+    than the batch has in use: 2048 tokens over about 1230 work items against a grid of 512 (group 4) or 1024
+    (group 2) records, so every workgroup walks two or three records.  Ranks 8, 16 and 32 in one pool (the rank-32
+    items take two shrink slices per workgroup), adapters with 64, 17 and 16 tokens next to 1200 with one or two,
+    tokens without an adapter; accumulate and delta against the oracle."""
+    rng = np.random.default_rng(4242)
+    N, T, hin, hout = 1200, 2048, 8192, 1024
+    ranks = rng.choice([8, 16, 32], N)
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=FP16)
+    ids = rng.permutation(N)
+    rest = T - 148 - (N - 3)                                      # tokens left after one per remaining adapter
+    tok = np.concatenate([np.repeat(ids[0], 64), np.repeat(ids[1], 17), np.repeat(ids[2], 16), np.full(51, -1),
+                          ids[3:], ids[3:3 + rest]]).astype(np.int32)
+    assert len(tok) == T
+    tok = rng.permutation(tok)
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), FP16)
+    y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), FP16)
+    say(f"bgmv many-round launch, T={T}, {N} adapters of rank 8/16/32, group={group}")
+    got = _run(pp, x, tok, y0, group, accumulate=True, fused=False)
+    assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16, "accumulate")
+    got = _run(pp, x, tok, None, group, accumulate=False, fused=False)
+    want = oracle_apply(pp, x, tok, None)
+    assert_close_bits(got, want, FP16, "delta")
+    assert not np.any(f32_of(got, FP16)[tok < 0]), "rows of tokens without an adapter must be zeros in y = delta mode"
