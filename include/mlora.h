@@ -179,6 +179,10 @@ int mlora_assist_import(int n_proj, void *const *res, const void *const *out_slo
  * fused launch.  workspace == NULL selects the fused launch.  Calls that share a workspace must be
  * ordered on one stream.  Both forms accumulate in fp32 and
  * round once; they differ only in the order the fp32 partial sums of the shrink are added.
+ * When the batch makes for many rounds of workgroups (thousands of slices), the two launches cover fewer
+ * records than MLORA_WORK_CAP(T): a workgroup serves records b, b + stride, ... of its residue mod 8 and stops
+ * at the first empty one.  The layout mlora_pool_gather writes (records in use of each residue first) is what
+ * makes that valid; a caller that fills `work` itself must keep it.
  */
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank);
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
