@@ -44,6 +44,7 @@ CASES = [
     ("fp16 hetero ranks 4096x4096", [40, 100, 7, 64, 129], [8, 16, 32, 64, 24], 4096, 4096, FP16),
     ("rank 16 pool 1024x2048", [63, 64, 65, 1], [16, 8, 16, 3], 1024, 2048, FP16),
     ("odd widths 200x72 bf16", [5, 70], [32, 5], 200, 72, BF16),
+    ("tile boundaries 127/128/129 r32 2048x1024", [127, 128, 129, 63, 64, 65], [32, 32, 16, 32], 2048, 1024, FP16),
 ]
 
 
