@@ -15,6 +15,14 @@
 // of eight (one per XCD) with the slices and projections of those eight in between, so the
 // records in use come first in launch order and the empty tail costs no waiting.
 //
+// The kernels come in two instantiations, chosen by the host from the size of the batch (launch_sliced):
+//   BIG = false, a launch of about one round of workgroups (hundreds to a few thousand slices): one workgroup
+//     per (record, projection, slice) over the host's upper bound on the records, nontemporal row loads; what
+//     counts is the chain of dependent loads of one workgroup;
+//   BIG = true, a launch of many rounds (config 5: 8000 shrink slices): the grid covers fewer records and a
+//     workgroup walks records b, b + stride, ..., a rank-32 item takes two shrink slices per workgroup, rows are
+//     read with ordinary loads, the record header as constant memory; what counts is throughput.
+//
 // Replaces punica.ops.add_lora_bgmv as called from lightllm/models/lora_gpu.py:138,150,162.
 #include <type_traits>
 #include "mlora_args.hpp"
