@@ -351,29 +351,39 @@ def test_bgmv_config5_one_layer_full_pool():
         assert torch.allclose(ys[p].float(), want[p][o], rtol=RTOL, atol=ATOL), p
 
 
-@pytest.mark.parametrize("group", [4, 2])
-def test_bgmv_many_round_launch_walks_several_records(group):
-    """A launch of many rounds of workgroups (here 8 shrink slices x 1700 possible records) covers fewer records
-    than the batch has in use: 2048 tokens over about 1230 work items against a grid of 512 (group 4) or 1024
-    (group 2) records, so every workgroup walks two or three records.  Ranks 8, 16 and 32 in one pool (the rank-32
-    items take two shrink slices per workgroup), adapters with 64, 17 and 16 tokens next to 1200 with one or two,
-    tokens without an adapter; accumulate and delta against the oracle."""
-    rng = np.random.default_rng(4242)
-    N, T, hin, hout = 1200, 2048, 8192, 1024
-    ranks = rng.choice([8, 16, 32], N)
-    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=FP16)
+MANY_ROUNDS = [
+    # group, ranks in the pool, hin, T, adapters, dtype: each makes >= 16 rounds of shrink workgroups by the host's
+    # count (slices of hin x min(T/group + adapters + 1, T rounded up to 8) records >= 16 x 768)
+    (4, [8, 16, 32], 8192, 2048, 1200, FP16),
+    (2, [8, 16, 32], 8192, 2048, 1200, FP16),
+    (1, [16, 64], 8192, 2048, 600, BF16),
+    (8, [8, 16], 16384, 4096, 1200, BF16),
+]
+
+
+@pytest.mark.parametrize("group,rank_set,hin,T,N,dtype", MANY_ROUNDS, ids=[f"g{c[0]}-r{max(c[1])}-{c[2]}" for c in MANY_ROUNDS])
+def test_bgmv_many_round_launch_walks_several_records(group, rank_set, hin, T, N, dtype):
+    """A launch of many rounds of workgroups (thousands of possible (record, slice) pairs) covers fewer records
+    than the batch has in use, so every workgroup walks several records.  Mixed ranks in one pool (in a rank-32
+    launch the rank-32 items take two shrink slices per workgroup), adapters with 64, 17 and 16 tokens next to
+    hundreds with one to three, tokens without an adapter; accumulate and delta against the oracle, for each launch
+    width (rank 16 / 32 / 64), token group and both dtypes."""
+    rng = np.random.default_rng(4242 + group)
+    hout = 1024
+    ranks = rng.choice(rank_set, N)
+    pp = PagedPool(rng, ranks, hin, hout, page_rows=8, dtype=dtype)
     ids = rng.permutation(N)
     rest = T - 148 - (N - 3)                                      # tokens left after one per remaining adapter
     tok = np.concatenate([np.repeat(ids[0], 64), np.repeat(ids[1], 17), np.repeat(ids[2], 16), np.full(51, -1),
-                          ids[3:], ids[3:3 + rest]]).astype(np.int32)
+                          ids[3:], rng.choice(ids[3:], rest)]).astype(np.int32)
     assert len(tok) == T
     tok = rng.permutation(tok)
-    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), FP16)
-    y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), FP16)
-    say(f"bgmv many-round launch, T={T}, {N} adapters of rank 8/16/32, group={group}")
+    x = bits_of(rng.standard_normal((T, hin)).astype(np.float32), dtype)
+    y0 = bits_of(rng.standard_normal((T, hout)).astype(np.float32), dtype)
+    say(f"bgmv many-round launch, T={T}, {N} adapters of rank {rank_set}, hin={hin}, group={group}")
     got = _run(pp, x, tok, y0, group, accumulate=True, fused=False)
-    assert_close_bits(got, oracle_apply(pp, x, tok, y0), FP16, "accumulate")
+    assert_close_bits(got, oracle_apply(pp, x, tok, y0), dtype, "accumulate")
     got = _run(pp, x, tok, None, group, accumulate=False, fused=False)
     want = oracle_apply(pp, x, tok, None)
-    assert_close_bits(got, want, FP16, "delta")
-    assert not np.any(f32_of(got, FP16)[tok < 0]), "rows of tokens without an adapter must be zeros in y = delta mode"
+    assert_close_bits(got, want, dtype, "delta")
+    assert not np.any(f32_of(got, dtype)[tok < 0]), "rows of tokens without an adapter must be zeros in y = delta mode"
