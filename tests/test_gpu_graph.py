@@ -103,3 +103,54 @@ def test_graph_replays_of_the_one_pass_projection_match_eager():
         torch.cuda.synchronize()
         assert scratch.isfinite()
         assert torch.equal(y, want), rep
+
+
+@pytest.mark.parametrize("size", ["one round (config 2 shape)", "many rounds (config 5 layer)"])
+def test_graph_replay_follows_a_changed_batch(size):
+    """A captured decode step (gather + BGMV) reads its token -> adapter vector from device memory: when the caller
+    overwrites that vector between replays, the replay must use the new grouping -- the work records are rewritten by
+    the gather node and read by the decode kernels of the same replay (header words through scalar loads), so a stale
+    copy anywhere would show here.  Each replay is compared bit for bit with an eager run on the same batch."""
+    from mlora import workloads
+    if size.startswith("one"):
+        shapes, T, N, rank, alpha = workloads.LLAMA7B_ATTN, 256, 64, 16, 1.0
+    else:
+        shapes, T, N, rank, alpha = workloads.LLAMA7B_ALL, 512, 1000, 32, 1.1
+    names = list(shapes)
+    wl = workloads.make_decode("graph", shapes, 1, T, N, [rank], alpha, seed=77, device="cuda")
+    pool = wl.pool
+    rng = np.random.default_rng(5)
+    batches = [wl.tok_adapter,
+               workloads.zipf_adapters(rng, T, N, 0.6),
+               np.where(rng.random(T) < 0.1, -1, workloads.zipf_adapters(rng, T, N, 1.4)).astype(np.int32)]
+    tok = torch.from_numpy(batches[0].copy()).cuda()
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    xs = {h: torch.randn(T, h, device="cuda", generator=gen).half() for h in {s[0] for s in shapes.values()}}
+    y0 = [torch.randn(T, shapes[p][1], device="cuda", generator=gen).half() for p in names]
+    ys = [t.clone() for t in y0]
+    plan = plan_decode(tok, pool, group=4)
+
+    def step():
+        for y, src in zip(ys, y0):
+            y.copy_(src)
+        plan_decode(tok, pool, out=plan)
+        bgmv(ys, [xs[shapes[p][0]] for p in names], pool, 0, names, tok, plan=plan, fused=False)
+
+    want = []
+    for bt in batches:
+        tok.copy_(torch.from_numpy(bt))
+        step()
+        torch.cuda.synchronize()
+        want.append([t.clone() for t in ys])
+    assert not torch.equal(want[0][0], want[1][0])
+    tok.copy_(torch.from_numpy(batches[0]))
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for rep, which in enumerate([0, 1, 2, 1, 0, 2]):
+        tok.copy_(torch.from_numpy(batches[which]))
+        say(f"graph ({size}): replay {rep} on batch {which}")
+        g.replay()
+        torch.cuda.synchronize()
+        for got, w in zip(ys, want[which]):
+            assert torch.equal(got, w), (rep, which)
