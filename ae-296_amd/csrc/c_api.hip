@@ -559,13 +559,11 @@ SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
 {
     SgmvWs w;
     w.max_tiles = T / SG_TM + 2 * n_seg + 1;       // aligned cuts can add one partial tile at either end of a segment
-    // shrink workgroups: about three per CU for a single projection; a call over several projections
-    // has that many already with fewer splits, and fewer splits mean less partial-sum traffic
+    // shrink workgroups: about three per CU for a single projection; a call over several projections has about
+    // that many with one or two splits already (one workgroup serves the projections that share x), and fewer
+    // splits mean less partial-sum traffic (swept 512 .. 4096 on configs 4 and 5: 768 - 1024 is the flat optimum)
     const long long per_split = (long long)w.max_tiles * n_proj;
-#ifndef MLORA_SG_TARGET
-#define MLORA_SG_TARGET 2048
-#endif
-    const long long target = n_proj > 1 ? MLORA_SG_TARGET : 768;
+    const long long target = n_proj > 1 ? 1024 : 768;
     long long ks = (target + per_split - 1) / per_split;
     w.ksplit = ks < 1 ? 1 : (ks > 8 ? 8 : (int)ks);
     // a projection with a longer K than the others of its call gets proportionally more splits (up to three
@@ -606,19 +604,16 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
         int ks = (int)(((long long)w.ksplit * a.pr[p].hin + hin_min / 2) / (hin_min > 0 ? hin_min : 1));
         a.pr[p].ksplit = ks < w.ksplit ? w.ksplit : (ks > w.ks_cap ? w.ks_cap : ks);
         // 512 columns per expand workgroup amortise the V operand; fewer when that leaves the chip idle
-#ifndef MLORA_SG_COLS
-#define MLORA_SG_COLS 512
-#endif
-        int cols = MLORA_SG_COLS;
+        int cols = 512;
         if (a.n_proj == 1)
             while (cols > 128 && (long long)w.max_tiles * ((a.pr[p].hout + cols - 1) / cols) < 1024) cols >>= 1;
         a.pr[p].cols = cols;
         a.pr[p].ncb = (a.pr[p].hout + cols - 1) / cols;
     }
-    // shrink groups: consecutive projections that read the same activations
+    // shrink groups: up to three consecutive projections that read the same activations (one workgroup serves a group)
     a.n_grp = 0;
     for (int p = 0; p < a.n_proj; p++) {
-        if (p > 0 && a.pr[p].x == a.pr[p - 1].x && a.pr[p].hin == a.pr[p - 1].hin) a.grp_n[a.n_grp - 1]++;
+        if (p > 0 && a.pr[p].x == a.pr[p - 1].x && a.pr[p].hin == a.pr[p - 1].hin && a.grp_n[a.n_grp - 1] < 3) a.grp_n[a.n_grp - 1]++;
         else { a.grp_first[a.n_grp] = p; a.grp_n[a.n_grp] = 1; a.n_grp++; }
     }
 }

@@ -125,9 +125,9 @@ struct SgmvProj {
 struct SgmvArgs {
     SgmvProj pr[MAX_PROJ];
     int n_proj;
-    // Shrink launch: consecutive projections that read the same x form a group; the workgroups of a
-    // group's members that cover the same tokens and K split run back to back on one XCD, so x comes
-    // from HBM once per group.  grp_end[g] = first workgroup id after group g.
+    // Shrink launch: up to three consecutive projections that read the same x form a group, served by one
+    // workgroup per (tile, K split): x comes from HBM once per group and is multiplied with every member's A.
+    // grp_end[g] = first workgroup id after group g.
     int n_grp;
     int grp_first[MAX_PROJ], grp_n[MAX_PROJ];
     unsigned grp_end[MAX_PROJ];

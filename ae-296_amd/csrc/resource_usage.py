@@ -40,7 +40,8 @@ LIMITS = [
     ("bgmv_split.hip", r"bgmv_expand_kernel<\d, [124], 32, 128, 256, false>", {"occupancy": (3, 8)}),
     ("bgmv_decode.hip", r".", {"scratch": (0, 0), "vgpr_spill": (0, 0)}),
     ("sgmv_prefill.hip", r".", {"scratch": (0, 0), "vgpr_spill": (0, 0)}),
-    ("sgmv_prefill.hip", r"sgmv_shrink_kernel<", {"occupancy": (3, 8)}),
+    ("sgmv_prefill.hip", r"sgmv_shrink_kernel<\d, (16|32)>", {"occupancy": (3, 8)}),
+    ("sgmv_prefill.hip", r"sgmv_shrink_kernel<\d, 64>", {"occupancy": (2, 8)}),
 ]
 
 FIELDS = {"TotalSGPRs": "sgprs", "VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch",

@@ -67,19 +67,6 @@ __device__ __forceinline__ bool xcd_remap(int w, int n_second, int &tile, int &s
     tile = run * XRUN + i;
     return true;
 }
-// Shrink form: `second` is (K split, member of the projection group) with the member varying faster and
-// the XCD chosen by the split alone, so the members that read the same x slice follow each other on one XCD.
-__device__ __forceinline__ void xcd_remap_group(int w, int n_split, int n_member, int &tile, int &split, int &member)
-{
-    const int r = w & 7, slot = w >> 3;
-    const int i = slot % XRUN;
-    const int s2 = (slot / XRUN) % (n_split * n_member);
-    const int j = slot / (XRUN * n_split * n_member);
-    split = s2 / n_member;
-    member = s2 - split * n_member;
-    const int run = ((r - split) & 7) + 8 * j;
-    tile = run * XRUN + i;
-}
 __host__ __device__ inline long long xcd_grid(int max_tiles, int n_second)
 {
     const long long runs = (max_tiles + XRUN - 1) / XRUN;
@@ -184,29 +171,33 @@ __device__ __forceinline__ float4_t mfma16(const uint4 &a, const uint4 &b, float
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf168_t, a), __builtin_bit_cast(bf168_t, b), c, 0, 0, 0);
 }
 
+constexpr int SG_NM = 3;     // projections of one x that a shrink workgroup serves (a larger group is cut by the host)
+
 template <int DT, int RMAX>
 __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
 {
-    // One workgroup: 64 tokens x RMAX ranks over one K slice.  A stage is 128 columns: the X tile
-    // (64 rows x 256 B) and the A tile (RMAX rows x 256 B) are read with 16-byte loads in which every
-    // 16-lane row covers 256 contiguous bytes, parked in LDS, and consumed from there as MFMA operands
-    // (8 contiguous K values per lane).  The next stage's loads are in flight while this one computes.
+    // One workgroup: 64 tokens x RMAX ranks over one K slice, for every projection of its group (up to SG_NM
+    // projections that read the same x: q, k, v; gate, up).  A stage is 128 columns: the X tile (64 rows x 256 B)
+    // and one A tile per projection (RMAX rows x 256 B) are read with 16-byte loads in which every 16-lane row
+    // covers 256 contiguous bytes, parked in LDS, and consumed from there as MFMA operands (8 contiguous K
+    // values per lane); the X operand of a step is read from LDS once and multiplied with every projection's A.
+    // The next stage's loads are in flight while this one computes.  x is fetched once per group (streaming).
     constexpr int NB = RMAX / 16;            // rank blocks of 16
     constexpr int KB = 128;                  // columns per stage
     constexpr int CPR = KB / 8;              // 16-byte chunks per row and stage
     constexpr int PITCH = KB * 2 + 32;       // LDS row pitch in bytes; the padding spreads the operand reads over the banks
                                              // (measured: no padding 2x slower, 16 bytes 6 % slower than 32, 48..144 slower again)
     constexpr int XP = TM * CPR / SG_NT;     // X loads per thread and stage (4)
-    constexpr int AP = (RMAX * CPR + SG_NT - 1) / SG_NT;   // A loads per thread and stage (1, 2 or 4)
+    constexpr int AP = (RMAX * CPR + SG_NT - 1) / SG_NT;   // A loads per thread, projection and stage (1, 2 or 4)
     __shared__ __attribute__((aligned(16))) unsigned char s_x[TM * PITCH];
-    __shared__ __attribute__((aligned(16))) unsigned char s_a[RMAX * PITCH];
+    __shared__ __attribute__((aligned(16))) unsigned char s_a[SG_NM][RMAX * PITCH];
     int grp = 0;
     while (grp + 1 < p.n_grp && blockIdx.x >= p.grp_end[grp]) grp++;
-    int tile, split, member;
-    xcd_remap_group((int)(blockIdx.x - (grp ? p.grp_end[grp - 1] : 0u)), p.pr[p.grp_first[grp]].ksplit, p.grp_n[grp],
-                    tile, split, member);
-    const SgmvProj &pj = p.pr[p.grp_first[grp] + member];
-    const bool shared_x = p.grp_n[grp] > 1;
+    int tile, split;
+    const int nm = p.grp_n[grp] < SG_NM ? p.grp_n[grp] : SG_NM; // projections this workgroup serves
+    xcd_remap((int)(blockIdx.x - (grp ? p.grp_end[grp - 1] : 0u)), p.pr[p.grp_first[grp]].ksplit, tile, split);
+    const int p0 = p.grp_first[grp];
+    const SgmvProj &pj = p.pr[p0];
     if (tile >= p.n_tiles[0]) return;
     const int32_t *__restrict__ rec = p.tile_rec + (size_t)tile * TILE_WORDS;
     const int ntok = rec[0], adapter = rec[1];
@@ -219,7 +210,6 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
 
     const int hin = pj.hin;
     const uint16_t *__restrict__ x = static_cast<const uint16_t *>(pj.x);
-    const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(pj.a_rows);
     const int lrow = tid >> 4, lchk = tid & 15;                // this thread's row (per pass of 16) and chunk
     const uint4 *xp[XP];
 #pragma unroll
@@ -228,36 +218,44 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
         t = t < ntok ? t : ntok - 1;                            // tail rows repeat the last token; never stored
         xp[q] = reinterpret_cast<const uint4 *>(x + (size_t)(tok0 + t) * hin);
     }
-    const uint4 *ap[AP];
+    const uint4 *ap[SG_NM][AP];
 #pragma unroll
-    for (int q = 0; q < AP; q++) {
-        const int j = lrow + 16 * q;
-        const int row = j < RMAX ? rows[j] : -1;
-        ap[q] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+    for (int mm = 0; mm < SG_NM; mm++) {
+        const uint16_t *arows = static_cast<const uint16_t *>(p.pr[p0 + (mm < nm ? mm : 0)].a_rows);
+#pragma unroll
+        for (int q = 0; q < AP; q++) {
+            const int j = lrow + 16 * q;
+            const int row = j < RMAX ? rows[j] : -1;
+            ap[mm][q] = reinterpret_cast<const uint4 *>(arows + (size_t)(row >= 0 ? row : 0) * hin);
+        }
     }
-    float4_t acc[NB];
+    float4_t acc[SG_NM][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) acc[nb] = float4_t{0.f, 0.f, 0.f, 0.f};
+    for (int mm = 0; mm < SG_NM; mm++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++) acc[mm][nb] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     const int ncc = hin >> 3;                                   // 16-byte chunks per row
     const int nstage = (ncc + CPR - 1) / CPR;
     const int per = (nstage + pj.ksplit - 1) / pj.ksplit;
     const int st0 = split * per;
     const int st1 = st0 + per < nstage ? st0 + per : nstage;
-    uint4 xr[XP], ar[AP];
+    uint4 xr[XP], ar[SG_NM][AP];
     auto load_stage = [&](int st) {
         const int c = st * CPR + lchk;
         const bool ok = c < ncc;                                // K tail: both operands become zero
         const int cs = ok ? c : ncc - 1;
 #pragma unroll
         for (int q = 0; q < XP; q++) {
-            // x read by one projection only passes through once (streaming hint); x shared by the members
-            // of a group must stay in L2 for the next member
-            xr[q] = shared_x ? ldg16(xp[q] + cs) : ldg16_stream(xp[q] + cs);
+            xr[q] = ldg16_stream(xp[q] + cs);                   // x passes through once per group
             if (!ok) xr[q] = zero16();
         }
 #pragma unroll
-        for (int q = 0; q < AP; q++) { ar[q] = ldg16(ap[q] + cs); if (!ok) ar[q] = zero16(); }
+        for (int mm = 0; mm < SG_NM; mm++)
+            if (mm < nm) {
+#pragma unroll
+                for (int q = 0; q < AP; q++) { ar[mm][q] = ldg16(ap[mm][q] + cs); if (!ok) ar[mm][q] = zero16(); }
+            }
     };
     if (st0 < st1) load_stage(st0);
 #pragma unroll 1
@@ -267,32 +265,44 @@ __global__ __launch_bounds__(SG_NT) void sgmv_shrink_kernel(const SgmvArgs p)
         for (int q = 0; q < XP; q++)
             *reinterpret_cast<uint4 *>(s_x + (lrow + 16 * q) * PITCH + lchk * 16) = xr[q];
 #pragma unroll
-        for (int q = 0; q < AP; q++)
-            if (lrow + 16 * q < RMAX) *reinterpret_cast<uint4 *>(s_a + (lrow + 16 * q) * PITCH + lchk * 16) = ar[q];
+        for (int mm = 0; mm < SG_NM; mm++)
+            if (mm < nm) {
+#pragma unroll
+                for (int q = 0; q < AP; q++)
+                    if (lrow + 16 * q < RMAX) *reinterpret_cast<uint4 *>(s_a[mm] + (lrow + 16 * q) * PITCH + lchk * 16) = ar[mm][q];
+            }
         __syncthreads();
         if (st + 1 < st1) load_stage(st + 1);
 #pragma unroll
         for (int ks = 0; ks < KB / 32; ks++) {
             const uint4 xf = *reinterpret_cast<const uint4 *>(s_x + (wave * 16 + m) * PITCH + (ks * 4 + g) * 16);
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) {
-                const uint4 af = *reinterpret_cast<const uint4 *>(s_a + (nb * 16 + m) * PITCH + (ks * 4 + g) * 16);
-                acc[nb] = mfma16<DT>(xf, af, acc[nb]);
-            }
+            for (int mm = 0; mm < SG_NM; mm++)
+                if (mm < nm) {
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++) {
+                        const uint4 af = *reinterpret_cast<const uint4 *>(s_a[mm] + (nb * 16 + m) * PITCH + (ks * 4 + g) * 16);
+                        acc[mm][nb] = mfma16<DT>(xf, af, acc[mm][nb]);
+                    }
+                }
         }
     }
     // D[token 4g+i][rank m] per 16x16 block; rank columns that do not exist are stored as zero.
-    float *vout = pj.v + ((size_t)split * p.T + tok0 + wave * 16) * VSTRIDE;
 #pragma unroll
-    for (int nb = 0; nb < NB; nb++) {
-        const int col = nb * 16 + m;
-        const bool col_ok = rows[col] >= 0;
+    for (int mm = 0; mm < SG_NM; mm++)
+        if (mm < nm) {
+            float *vout = p.pr[p0 + mm].v + ((size_t)split * p.T + tok0 + wave * 16) * VSTRIDE;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int trow_o = wave * 16 + 4 * g + i;
-            if (trow_o < ntok) vout[(size_t)(4 * g + i) * VSTRIDE + col] = col_ok ? acc[nb][i] : 0.f;
+            for (int nb = 0; nb < NB; nb++) {
+                const int col = nb * 16 + m;
+                const bool col_ok = rows[col] >= 0;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int trow_o = wave * 16 + 4 * g + i;
+                    if (trow_o < ntok) vout[(size_t)(4 * g + i) * VSTRIDE + col] = col_ok ? acc[mm][nb][i] : 0.f;
+                }
+            }
         }
-    }
 }
 
 // ------------------------------------------------------------------ reduce
@@ -562,7 +572,7 @@ static int launch_rmax(const SgmvArgs &a, int phases, hipStream_t s)
     SgmvArgs g = a;
     unsigned end = 0;
     for (int q = 0; q < g.n_grp; q++) {
-        end += (unsigned)xcd_grid(g.max_tiles, g.pr[g.grp_first[q]].ksplit * g.grp_n[q]);
+        end += (unsigned)xcd_grid(g.max_tiles, g.pr[g.grp_first[q]].ksplit);
         g.grp_end[q] = end;
     }
     const unsigned sgrid = end;
