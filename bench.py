@@ -44,6 +44,7 @@ MIN_LEG_MS = 100.0                  # every leg is repeated until its timed regi
 # the figures live in the committed profile summaries, one `key: value` line each, and are read from there.
 TRAFFIC_SOURCE = {
     "c2": ("profiles/bgmv_c2_bench.txt", "hbm_bytes_per_decode_call"),
+    "c3": ("profiles/bgmv_c3_bench.txt", "hbm_bytes_per_decode_call"),
     "c4": ("profiles/sgmv_c4_bench.txt", "hbm_bytes_per_step"),
     "c5": ("profiles/mixed_c5_bench.txt", "hbm_bytes_per_decode_call"),
 }
@@ -804,7 +805,7 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
                                      "frac": alg_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                      "algorithmic_bytes_per_step": alg_step, "prefill_bytes_per_layer": alg_pre,
                                      "kernels": "gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"}})
-    traffic, src = traffic_of(workload, group == 4 and L == cfg["layers"] and not fused)
+    traffic, src = traffic_of(workload, group == mlora.ops.default_group(cfg["T"]) and L == cfg["layers"] and not fused)
 
     out = {
         "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",
