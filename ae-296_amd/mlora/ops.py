@@ -148,11 +148,14 @@ def side_by_side(side: SideStream, on_side, on_main) -> None:
     main = torch.cuda.current_stream()
     side.fork.record(main)
     side.stream.wait_event(side.fork)
-    with torch.cuda.stream(side.stream):
-        on_side()
-    on_main()
-    side.join.record(side.stream)
-    main.wait_event(side.join)
+    try:
+        with torch.cuda.stream(side.stream):
+            on_side()
+        on_main()
+    finally:
+        # joined also when a half raised: work already queued on the side stream stays ordered before what follows
+        side.join.record(side.stream)
+        main.wait_event(side.join)
 
 
 # ---------------------------------------------------------------------- decode
