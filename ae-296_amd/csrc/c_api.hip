@@ -607,8 +607,16 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
         int cols = 512;
         if (a.n_proj == 1)
             while (cols > 128 && (long long)w.max_tiles * ((a.pr[p].hout + cols - 1) / cols) < 1024) cols >>= 1;
+        // ... and a block count per tile that the tile-major order of the expand can use (a multiple of eight or just
+        // below one): otherwise the width that gives the nearest multiple of eight blocks, in whole cache lines
+        int ncb = (a.pr[p].hout + cols - 1) / cols;
+        if (!mlora::tile_major(ncb) && ncb >= 6) {
+            const int n8 = ((ncb + 3) / 8) * 8 > 0 ? ((ncb + 3) / 8) * 8 : 8;
+            const int c8 = ((a.pr[p].hout + n8 - 1) / n8 + 63) / 64 * 64;
+            if (c8 >= 256 && c8 <= 1024 && mlora::tile_major((a.pr[p].hout + c8 - 1) / c8)) { cols = c8; ncb = (a.pr[p].hout + c8 - 1) / c8; }
+        }
         a.pr[p].cols = cols;
-        a.pr[p].ncb = (a.pr[p].hout + cols - 1) / cols;
+        a.pr[p].ncb = ncb;
     }
     // shrink groups: up to three consecutive projections that read the same activations (one workgroup serves a group)
     a.n_grp = 0;

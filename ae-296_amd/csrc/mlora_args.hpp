@@ -108,6 +108,10 @@ struct GatherArgs {
     int32_t *counters;
 };
 
+// Whether a projection with `ncb` column blocks per tile runs its expand workgroups tile-major (the blocks of a
+// tile numbered up to the next multiple of eight): only when at most an eighth of the numbers stays unused.
+__host__ __device__ inline bool tile_major(int ncb) { return (((ncb + 7) & ~7) - ncb) * 8 <= ncb; }
+
 // One projection of a prefill call.
 struct SgmvProj {
     void *y;
