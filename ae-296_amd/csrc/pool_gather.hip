@@ -237,9 +237,10 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
             ch_idx++;
         }
     }
-    // ---- decode work records, in launch order: workgroup b of a projection reads record b.
-    // Consecutive chunks go to the same XCD (workgroups are dealt to the 8 XCDs round-robin).  Batches
-    // beyond 2048 tokens (chunk headers not in LDS) keep plain chunk order.
+    // ---- decode work records, in launch order: the records in use first; records b, b + 8, ... hold consecutive
+    // chunks (the one-launch decode form, whose workgroup b of a projection reads record b, runs them on one XCD:
+    // workgroups are dealt to the 8 XCDs round-robin; the two-launch form takes the records in order).  Batches
+    // beyond 2048 tokens (chunk headers not in LDS) keep plain chunk order inside each range.
     if (g.work) {
         __shared__ int s_nchunks;
         if (tid == GATHER_NT - 1) s_nchunks = ch_incl;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         const int n_chunks = s_nchunks;
         const int per_xcd = (n_chunks + 7) >> 3;
         if constexpr (LDS_HDR) {
-            // Within the range of chunks that goes to one XCD the records are written in order of falling rank
+            // Within each of the eight ranges of chunks the records are written in order of falling rank
             // (ties keep chunk order, so the chunks of one adapter stay next to each other): the workgroups of
             // the wide items are then dispatched first and the narrow ones fill in behind them.  A counting sort:
             // chunks per (XCD, rank), then one thread per (XCD, rank) places its chunks.

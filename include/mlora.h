@@ -91,10 +91,12 @@ int mlora_version(void);
  *   counters [MLORA_CNT_WORDS]
  *   work [MLORA_WORK_CAP(T) * MLORA_WORK_WORDS]  (optional, may be NULL) the chunks as decode work
  *                       records in launch order: position c of the chunk list is record
- *                       (c mod P) * 8 + c / P with P = ceil(n_chunks / 8), so a range of P consecutive
- *                       chunks runs on one XCD.  For T <= 2048 the chunks of each such range are placed by
- *                       falling rank (ties in chunk order), which starts the workgroups of wide items
- *                       first; the chunk_* arrays keep chunk order.  Record words:
+ *                       (c mod P) * 8 + c / P with P = ceil(n_chunks / 8): the records in use come first,
+ *                       records b, b + 8, ... hold a range of P consecutive chunks (the one-launch decode
+ *                       form runs such a range on one XCD; the two-launch form takes the records in
+ *                       order).  For T <= 2048 the chunks of each such range are placed by falling rank
+ *                       (ties in chunk order), which starts the workgroups of wide items first; the
+ *                       chunk_* arrays keep chunk order.  Record words:
  *                       [0] tokens (0 = empty record) [1] adapter [2] rank [3] scaling (float bits)
  *                       [4..11] token ids [12..15] 0 [16..79] row of rank row j in a rows slab, -1 if
  *                       j >= rank or the page id is outside [0, n_pages).
