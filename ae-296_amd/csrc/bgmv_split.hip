@@ -6,7 +6,7 @@
 // while every compute unit is pulling data.  The fused kernel's unit of work is a whole item
 // (an adapter's A and B rows for one projection, hundreds of KiB) and a decode batch has about
 // one item per compute unit, so a unit that gets two items finishes late and the others idle.
-// Here the unit of work is a 2048-column slice of an item (tens of KiB), there are several
+// Here the unit of work is a 1024- or 2048-column slice of an item (tens of KiB), there are several
 // slices per compute unit and per phase, and no row is fetched by more than one workgroup.
 // The price is the intermediate (T x slices x rank fp32, a few hundred KiB) going through L2.
 //
@@ -400,14 +400,17 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 
 // Slice sizes per rank bucket, in 16-byte chunks (8 columns): the bytes of a shrink workgroup grow
 // with rank x slice width, so wider ranks take narrower slices (measured over 64 / 128 / 256 chunks
-// on rank-16, rank-32, rank-64 and mixed-rank batches; 2048-column expand slices won everywhere).
+// on rank-16, rank-32, rank-64 and mixed-rank batches).  Expand slices: 2048 columns (256 threads) at
+// rank <= 16, 1024 columns (128 threads) above: with the record-major order of the workgroups the
+// narrower slices measured 2 % faster on the 512-token rank-32 batch and 1 % on the mixed-rank one
+// (512 columns the same, and 1024 at rank 16 2 % slower).
 template <int RMAX> struct Slices;
 template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
 #ifndef MLORA_KSC32
 #define MLORA_KSC32 128
 #endif
-template <> struct Slices<32> { static constexpr int KSC = MLORA_KSC32, NTE = 256; };
-template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 256; };
+template <> struct Slices<32> { static constexpr int KSC = MLORA_KSC32, NTE = 128; };
+template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 128; };
 // Sum over each aligned group of LPC lanes (1, 2, 4 or 8); every lane of the group gets the sum.
 template <int LPC>
 __device__ __forceinline__ float group_sum(float v)
@@ -578,7 +581,6 @@ static int launch_pair_bt(const BgmvArgs &a0, hipStream_t s)
     a.rec_stride_ex = record_stride<G>(a, a.ex_end[a.n_proj - 1], false);
     constexpr int RMAX = R <= 16 ? 16 : (R <= 32 ? 32 : 64);
     constexpr int KSC = Slices<RMAX>::KSC;
-    static_assert(Slices<RMAX>::NTE * 8 == 2048, "the transposed-B expand walks 2048-column slices");
     const long long n_sh = (long long)a.sh_end[a.n_proj - 1] * a.rec_stride_sh;
     const long long n_ex = (long long)a.ex_end[a.n_proj - 1] * a.rec_stride_ex;
     if (n_sh <= 0 || n_ex <= 0) return 0;
@@ -639,11 +641,12 @@ static int launch_sliced(const BgmvArgs &a, hipStream_t s)
     if (rounds >= 16) return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, true>(a, s);
     return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, false>(a, s);
 }
-void bgmv_split_slices(int max_rank, int *ksc, int *nte)
+void bgmv_split_slices(int max_rank, int *ksc, int *nte, bool transposed_b)
 {
     if (max_rank <= 16) { *ksc = Slices<16>::KSC; *nte = Slices<16>::NTE; }
     else if (max_rank <= 32) { *ksc = Slices<32>::KSC; *nte = Slices<32>::NTE; }
     else { *ksc = Slices<64>::KSC; *nte = Slices<64>::NTE; }
+    if (transposed_b) *nte = 256;              // bgmv_expand_bt_kernel walks 2048-column slices at every rank
 }
 
 template <int DT, int RMAX>

@@ -531,7 +531,7 @@ int mlora_bgmv_reflayout_multi(int n_proj, void *const *y, const void *const *x,
     if (workspace_bytes < need) return fail(MLORA_ENOSPACE, "workspace holds %lld bytes, %lld needed", (long long)workspace_bytes, (long long)need);
     a.vws = static_cast<float *>(workspace);
     int ksc, nte;
-    mlora::bgmv_split_slices(r, &ksc, &nte);
+    mlora::bgmv_split_slices(r, &ksc, &nte, true);
     a.ks_max = (max_hin + ksc * 8 - 1) / (ksc * 8);
     a.cs_max = (max_hout + nte * 8 - 1) / (nte * 8);
     int sh = 0, ex = 0;

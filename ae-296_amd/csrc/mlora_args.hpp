@@ -188,7 +188,7 @@ struct GemmLoraArgs {
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);   // a.b_transposed: max_rank is the pool's rank (8, 16, 32 or 64)
 int bgmv_split_rank_stride(int max_rank);
-void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks);   // slice widths in 16-byte chunks
+void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks, bool transposed_b = false);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);
 int launch_scatter(const ScatterArgs &a, hipStream_t s);
 int launch_assist_export(const AssistArgs &a, hipStream_t s);

@@ -37,7 +37,7 @@ LIMITS = [
     ("bgmv_split.hip", r"bgmv_shrink_kernel<\d, [124], 16, 256, false>", {"occupancy": (4, 8)}),
     ("bgmv_split.hip", r"bgmv_expand_kernel<\d, [124], 16, 256, 256, false>", {"occupancy": (3, 8)}),
     ("bgmv_split.hip", r"bgmv_shrink_kernel<\d, [124], 32, 128, false>", {"occupancy": (3, 8)}),
-    ("bgmv_split.hip", r"bgmv_expand_kernel<\d, [124], 32, 128, 256, false>", {"occupancy": (3, 8)}),
+    ("bgmv_split.hip", r"bgmv_expand_kernel<\d, [124], 32, 128, 128, false>", {"occupancy": (3, 8)}),
     ("bgmv_decode.hip", r".", {"scratch": (0, 0), "vgpr_spill": (0, 0)}),
     ("sgmv_prefill.hip", r".", {"scratch": (0, 0), "vgpr_spill": (0, 0)}),
     ("sgmv_prefill.hip", r"sgmv_shrink_kernel<\d, (16|32)>", {"occupancy": (3, 8)}),
