@@ -705,7 +705,7 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
     from mlora import workloads
 
     cfg = DECODE[workload]
-    group = args.group if args.group >= 0 else mlora.ops.default_group(cfg["T"])
+    group = args.group if args.group >= 0 else mlora.ops.group_for(cfg["T"], len(cfg["projs"]), cfg["N"])
     L = args.layers if args.layers > 0 else cfg["layers"]
     shapes = workloads.LLAMA7B_ATTN if cfg["shapes"] == "7b_attn" else workloads.LLAMA7B_ALL
     projs = cfg["projs"]
@@ -805,7 +805,7 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
                                      "frac": alg_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
                                      "algorithmic_bytes_per_step": alg_step, "prefill_bytes_per_layer": alg_pre,
                                      "kernels": "gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"}})
-    traffic, src = traffic_of(workload, group == mlora.ops.default_group(cfg["T"]) and L == cfg["layers"] and not fused)
+    traffic, src = traffic_of(workload, group == mlora.ops.group_for(cfg["T"], len(projs), cfg["N"]) and L == cfg["layers"] and not fused)
 
     out = {
         "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",

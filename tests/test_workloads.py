@@ -54,3 +54,12 @@ def test_decode_form_follows_the_batch_size():
     assert ops.decode_fused(128, 2, 3, 32) and not ops.decode_fused(192, 2, 3, 48)
     assert not ops.decode_fused(128, 2, 3, 128)          # every token its own adapter: 128 items per projection
     assert not ops.decode_fused(8, 4, 1, 8) and not ops.decode_fused(8, 8, 1, 8)
+
+
+def test_group_follows_the_launch_form_when_the_caller_names_its_projections():
+    from mlora import ops
+    # 128 tokens: three projections still run fused (2 tokens per item), seven run as the shrink + expand pair (4)
+    assert ops.group_for(128, 3, 32) == 2 and ops.group_for(128, 7, 128) == 4
+    # at 64 tokens and below the batch-size rule stands whatever the form; beyond 128 it is 4 anyway
+    assert ops.group_for(64, 7, 16) == 1 and ops.group_for(32, 1, 8) == 1
+    assert ops.group_for(256, 4, 64) == 4 and ops.group_for(512, 7, 1000) == 4
