@@ -71,12 +71,9 @@ __device__ __forceinline__ ItemId split_id(unsigned id, int nq)
 // Slices of the launch's width (Slices<RMAX>::KSC) that one shrink workgroup takes, by the rank bucket of
 // its item (more than 32, 17..32, 9..16, at most 8 rank rows): the bytes of a workgroup grow with
 // rank x width, so an item of low rank in a launch sized for rank 64 takes wider slices.
-#ifndef MLORA_F8BIG
-#define MLORA_F8BIG 2
-#endif
 template <int RMAX, bool BIG> struct SliceFactor;
 template <bool BIG> struct SliceFactor<16, BIG> { static constexpr int F16 = 1, F8 = 1, F4 = 1, F2 = 1; };
-template <bool BIG> struct SliceFactor<32, BIG> { static constexpr int F16 = 1, F8 = BIG ? MLORA_F8BIG : 1, F4 = 2, F2 = 4; };
+template <bool BIG> struct SliceFactor<32, BIG> { static constexpr int F16 = 1, F8 = BIG ? 2 : 1, F4 = 2, F2 = 4; };
 template <bool BIG> struct SliceFactor<64, BIG> { static constexpr int F16 = 1, F8 = 1, F4 = 2, F2 = 4; };
 template <int RMAX, bool BIG>
 __device__ __forceinline__ int slice_factor(int r)
@@ -252,11 +249,7 @@ template <int DT, int G, int RMAX, int KSC, int NTE, bool BIG>
 __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 {
     constexpr int NT = NTE;                                    // one 16-byte chunk of the slice per thread
-#ifndef MLORA_EBW_BIG
-#define MLORA_EBW_BIG 8
-#endif
-    constexpr int EBW = BIG ? MLORA_EBW_BIG : 8;
-    constexpr int EB = RMAX < EBW ? RMAX : EBW;                 // B rank rows in flight per lane
+    constexpr int EB = RMAX < 8 ? RMAX : 8;                     // B rank rows in flight per lane
     __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
 
     const int tid = threadIdx.x;
@@ -406,10 +399,7 @@ __global__ __launch_bounds__(NTE) void bgmv_expand_kernel(const BgmvArgs p)
 // (512 columns the same, and 1024 at rank 16 2 % slower).
 template <int RMAX> struct Slices;
 template <> struct Slices<16> { static constexpr int KSC = 256, NTE = 256; };
-#ifndef MLORA_KSC32
-#define MLORA_KSC32 128
-#endif
-template <> struct Slices<32> { static constexpr int KSC = MLORA_KSC32, NTE = 128; };
+template <> struct Slices<32> { static constexpr int KSC = 128, NTE = 128; };
 template <> struct Slices<64> { static constexpr int KSC = 128, NTE = 128; };
 // Sum over each aligned group of LPC lanes (1, 2, 4 or 8); every lane of the group gets the sum.
 template <int LPC>
@@ -559,15 +549,13 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
 // dispatch alone, which is a tenth of a launch of thousands of slices.  The stride is never below ceil(T/G)
 // (that many records are in use whenever every token has an adapter entry) and large enough for the launch to
 // hold a few rounds of workgroups, so that small batches keep one workgroup per record.
-#ifndef MLORA_GRID_TARGET
-#define MLORA_GRID_TARGET 3072
-#endif
+constexpr int GRID_TARGET = 3072;                               // (record, slice) pairs a many-round launch covers at least
 template <int G>
 static int record_stride(const BgmvArgs &a, int slices, bool big)
 {
     if (!big) return a.items_cap;                               // about one round of workgroups: one per record
     long long want = (a.T + G - 1) / G;
-    const long long fill = (MLORA_GRID_TARGET + slices - 1) / slices;
+    const long long fill = (GRID_TARGET + slices - 1) / slices;
     want = want > fill ? want : fill;
     want = (want + 7) / 8 * 8;
     return want < a.items_cap ? (int)want : a.items_cap;
@@ -637,7 +625,7 @@ static int launch_sliced(const BgmvArgs &a, hipStream_t s)
 {
     // Rounds of shrink workgroups the launch may need (host's upper bound on the work items, three workgroups per
     // compute unit): from about sixteen on, the items of a much-used adapter no longer run side by side.
-    const long long rounds = (long long)a.sh_end[a.n_proj - 1] * a.items_cap / (3 * 256);
+    const long long rounds = (long long)a.sh_end[a.n_proj - 1] * a.items_cap / (3 * device_compute_units());
     if (rounds >= 16) return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, true>(a, s);
     return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, false>(a, s);
 }

@@ -95,6 +95,25 @@ int check_dims(int hin, int hout)
 
 }  // namespace
 
+namespace mlora {
+
+int device_compute_units()
+{
+    static std::mutex mu;
+    static int cus[SCRATCH_MAX_DEVICES] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SCRATCH_MAX_DEVICES) return 256;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!cus[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    }
+    return cus[dev];
+}
+
+}  // namespace mlora
+
 extern "C" {
 
 const char *mlora_last_error(void) { return g_err; }
@@ -175,16 +194,6 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
     while ((1 << a.page_shift) < page_rows) a.page_shift++;
     const int rc = mlora::launch_scatter(a, static_cast<hipStream_t>(stream));
     if (rc) return fail(MLORA_ELAUNCH, "scatter launch failed: %s", hipGetErrorString((hipError_t)rc));
-    return MLORA_OK;
-}
-
-int mlora_probe_stream(void *buf, int64_t bytes, int mode, void *stream)
-{
-    if (bytes < 0 || (mode != 0 && mode != 1)) return fail(MLORA_EINVAL, "bytes must be >= 0 and mode 0 (read) or 1 (read-modify-write)");
-    if (bytes == 0) return MLORA_OK;
-    if (!buf || !aligned16(buf)) return fail(MLORA_EALIGN, "buf must be a 16-byte aligned device pointer");
-    const int rc = mlora::launch_stream_probe(buf, bytes, mode, nullptr, static_cast<hipStream_t>(stream));
-    if (rc) return fail(MLORA_ELAUNCH, "probe launch failed: %s", hipGetErrorString((hipError_t)rc));
     return MLORA_OK;
 }
 
@@ -585,6 +594,25 @@ SgmvWs sgmv_layout(int T, int n_seg, int n_proj)
     return w;
 }
 
+// Columns of y one expand workgroup covers, and the column blocks per tile that follow from it.
+// 512 columns amortise the V operand; fewer when that leaves the chip idle (single-projection calls), and a block
+// count per tile that the tile-major order of the expand can use (a multiple of eight or just below one):
+// otherwise the width that gives the nearest multiple of eight blocks, in whole cache lines.
+int expand_block_cols(int n_proj, int max_tiles, int hout, int *ncb_out)
+{
+    int cols = 512;
+    if (n_proj == 1)
+        while (cols > 128 && (long long)max_tiles * ((hout + cols - 1) / cols) < 1024) cols >>= 1;
+    int ncb = (hout + cols - 1) / cols;
+    if (!mlora::tile_major(ncb) && ncb >= 6) {
+        const int n8 = ((ncb + 3) / 8) * 8 > 0 ? ((ncb + 3) / 8) * 8 : 8;
+        const int c8 = ((hout + n8 - 1) / n8 + 63) / 64 * 64;
+        if (c8 >= 256 && c8 <= 1024 && mlora::tile_major((hout + c8 - 1) / c8)) { cols = c8; ncb = (hout + c8 - 1) / c8; }
+    }
+    if (ncb_out) *ncb_out = ncb;
+    return cols;
+}
+
 void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
 {
     char *base = static_cast<char *>(workspace);
@@ -603,18 +631,8 @@ void carve(mlora::SgmvArgs &a, void *workspace, const SgmvWs &w)
         a.pr[p].vlo = reinterpret_cast<uint16_t *>(pb + w.off_lo);
         int ks = (int)(((long long)w.ksplit * a.pr[p].hin + hin_min / 2) / (hin_min > 0 ? hin_min : 1));
         a.pr[p].ksplit = ks < w.ksplit ? w.ksplit : (ks > w.ks_cap ? w.ks_cap : ks);
-        // 512 columns per expand workgroup amortise the V operand; fewer when that leaves the chip idle
-        int cols = 512;
-        if (a.n_proj == 1)
-            while (cols > 128 && (long long)w.max_tiles * ((a.pr[p].hout + cols - 1) / cols) < 1024) cols >>= 1;
-        // ... and a block count per tile that the tile-major order of the expand can use (a multiple of eight or just
-        // below one): otherwise the width that gives the nearest multiple of eight blocks, in whole cache lines
-        int ncb = (a.pr[p].hout + cols - 1) / cols;
-        if (!mlora::tile_major(ncb) && ncb >= 6) {
-            const int n8 = ((ncb + 3) / 8) * 8 > 0 ? ((ncb + 3) / 8) * 8 : 8;
-            const int c8 = ((a.pr[p].hout + n8 - 1) / n8 + 63) / 64 * 64;
-            if (c8 >= 256 && c8 <= 1024 && mlora::tile_major((a.pr[p].hout + c8 - 1) / c8)) { cols = c8; ncb = (a.pr[p].hout + c8 - 1) / c8; }
-        }
+        int ncb = 0;
+        const int cols = expand_block_cols(a.n_proj, w.max_tiles, a.pr[p].hout, &ncb);
         a.pr[p].cols = cols;
         a.pr[p].ncb = ncb;
     }
@@ -634,6 +652,12 @@ int64_t mlora_sgmv_workspace_bytes(int T, int n_seg)
 {
     if (T <= 0 || n_seg <= 0) return 256;
     return (int64_t)sgmv_layout(T, n_seg, 1).total;
+}
+
+int mlora_sgmv_expand_cols(int T, int n_seg, int n_proj, int hout)
+{
+    if (T <= 0 || n_seg <= 0 || n_proj < 1 || n_proj > MLORA_MAX_PROJ || hout <= 0) return 0;
+    return expand_block_cols(n_proj, sgmv_layout(T, n_seg, n_proj).max_tiles, hout, nullptr);
 }
 
 int64_t mlora_sgmv_multi_workspace_bytes(int T, int n_seg, int n_proj)

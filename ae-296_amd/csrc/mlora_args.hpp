@@ -198,6 +198,7 @@ constexpr int SGMV_APPLY = 2;   // shrink, reduce, expand (the workspace already
 constexpr int SGMV_SHRINK = 4;  // the shrink launch alone: its partial sums feed the base GEMM + LoRA kernel
 int launch_sgmv(const SgmvArgs &a, int dtype, int max_rank, int phases, hipStream_t s);
 int launch_gemm_lora(const GemmLoraArgs &a, int dtype, int max_rank, hipStream_t s);
-int launch_stream_probe(void *p, long long bytes, int mode, unsigned *sink, hipStream_t s);
+// compute units of the current device (asked once per device; 256 when the query fails)
+int device_compute_units();
 
 }  // namespace mlora

@@ -2,8 +2,8 @@
 // the same run as the LoRA kernels so that their figures can be read against the box's own ceiling (which
 // differs from box to box and lies well under the published HBM peak).  MODE 0 reads every 16 bytes once with
 // the nontemporal loads the LoRA kernels use; MODE 1 reads, changes and writes back in place (the access
-// pattern of an accumulate-into-y expand).  No counterpart in the reference.
-#include "mlora_args.hpp"
+// pattern of an accumulate-into-y expand).  No counterpart in the reference.  Built into its own small library
+// (libmlora_probe.so) that only the benchmark loads: it is a measuring aid, not part of the operator surface.
 #include "mlora_dev.hpp"
 
 namespace mlora {
@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void stream_probe_kernel(uint4 *__restrict__ p
     if (MODE == 0 && acc == 0x9e3779b9u && sink) sink[0] = acc;      // keeps the loads alive; practically never taken
 }
 
-int launch_stream_probe(void *p, long long bytes, int mode, unsigned *sink, hipStream_t s)
+static int launch_stream_probe(void *p, long long bytes, int mode, unsigned *sink, hipStream_t s)
 {
     const long long n16 = bytes / 16;
     if (n16 <= 0) return 0;
@@ -43,3 +43,14 @@ int launch_stream_probe(void *p, long long bytes, int mode, unsigned *sink, hipS
 }
 
 }  // namespace mlora
+
+// One plain streaming pass over `bytes` of device memory at `buf` (16-byte aligned) on `stream`: mode 0 reads every
+// 16 bytes once, mode 1 adds 1 to the first 32-bit word of every 16 bytes in place.  Returns 0, -1 for a bad
+// argument, or the HIP error of the launch.
+extern "C" int mlora_probe_stream(void *buf, long long bytes, int mode, void *stream)
+{
+    if (bytes < 0 || (mode != 0 && mode != 1)) return -1;
+    if (bytes == 0) return 0;
+    if (!buf || (reinterpret_cast<uintptr_t>(buf) & 15u)) return -1;
+    return mlora::launch_stream_probe(buf, bytes, mode, nullptr, static_cast<hipStream_t>(stream));
+}

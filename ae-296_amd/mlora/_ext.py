@@ -40,7 +40,6 @@ SIGNATURES = {
     "mlora_pool_gather": (_i32, [_vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                  _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
     "mlora_pool_scatter": (_i32, [_i32, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i64, _i32, _vp]),
-    "mlora_probe_stream": (_i32, [_vp, _i64, _i32, _vp]),
     "mlora_host_alloc": (_i32, [_i64, _vp, _vp]),
     "mlora_host_free": (_i32, [_vp]),
     "mlora_assist_export": (_i32, [_vp, _i32, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
@@ -65,6 +64,7 @@ SIGNATURES = {
     "mlora_sgmv_planned": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32,
                                   _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     "mlora_sgmv_multi_workspace_bytes": (_i64, [_i32, _i32, _i32]),
+    "mlora_sgmv_expand_cols": (_i32, [_i32, _i32, _i32, _i32]),
     "mlora_sgmv_multi_planned": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32,
                                         _i32, _i32, _i64, _i32, _i32, _i32, _vp, _i64, _vp]),
     "mlora_gemm_lora_planned": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32,

@@ -49,12 +49,18 @@ class Lora_GPU:
         self.select_inds = [torch.randint(0, hi, (i + 1,), device=self.device, generator=self._gen)
                             for i in range(self.batch_size)]
         self._workspace = None
-        self._plan = None          # grouping of the current decode batch by adapter, and what it was made from
-        self._plan_key = None
-        self._qkv = None           # q, k, v deltas of the last decode input, and what they were computed from
-        self._qkv_key = None
-        self._ids = None           # int64 copy of the last int32 lora_ids
-        self._ids_key = None
+        # Grouping of the current decode batch by adapter.  It is served again only for the very tensor object it was
+        # made from (`_plan_src`, kept alive here so that neither its address nor its Python identity can pass to
+        # another tensor) at the same torch version counter: a serving loop builds `lora_ids` afresh every step
+        # (pre_process.py:50,100), and a new tensor of the same size often gets the freed one's address.
+        self._plan = None
+        self._plan_src = None
+        self._plan_ver = None
+        self._plan_gen = 0
+        self._qkv = None           # q, k, v deltas of the last decode input ...
+        self._qkv_x = None         # ... the input tensor itself (kept alive for the same reason) ...
+        self._qkv_w = []           # ... the six weight tensors ...
+        self._qkv_key = None       # ... and what else they were computed from
 
     def _rand(self, n, rows, cols):
         """[n, L, rows, cols] * 0.001, stored transposed and contiguous as the reference does."""
@@ -63,31 +69,40 @@ class Lora_GPU:
         return w.to(self.dtype).transpose(-1, -2).contiguous()
 
     # ------------------------------------------------------------------ apply
-    def _indices(self, bsz, lora_ids, device):
+    def _index_source(self, bsz, lora_ids):
         # The reference drops the request's adapter ids (``infer_state.lora_ids``, built at
         # pre_process.py:50,100) and applies a random stand-in; pass ``lora_ids`` to use the real ones.
         if lora_ids is None:
             return self.select_inds[bsz - 1]
         if lora_ids.numel() != bsz:
             raise ValueError("lora_ids must hold one adapter slot per row of x")
-        if lora_ids.dtype == torch.int64 and lora_ids.device == device:
-            return lora_ids
-        # int32 ids (pre_process.py:100) are widened once per distinct tensor contents, so that the three calls of a
-        # layer (and the layers of a step) see one index vector
-        key = (lora_ids.data_ptr(), lora_ids._version, str(lora_ids.device), lora_ids.dtype)
-        if self._ids_key != key:
-            self._ids, self._ids_key = lora_ids.to(device=device, dtype=torch.int64), key
-        return self._ids
+        return lora_ids
+
+    def _indices(self, bsz, lora_ids, device):
+        """The index vector as the kernels take it: int64 on the device (int32 ids, pre_process.py:100, are widened)."""
+        src = self._index_source(bsz, lora_ids)
+        if src.dtype == torch.int64 and src.device == device:
+            return src
+        return src.to(device=device, dtype=torch.int64)
 
     def plan_decode(self, bsz, lora_ids=None):
-        """Group the decode batch by adapter (one gather launch).  Called by ``invoke_one_layer_qkv`` when the index
-        vector is not the one the current plan was made from; a serving loop calls it once per step."""
-        device = self.q_down.device
-        cur_inds = self._indices(bsz, lora_ids, device)
+        """Group the decode batch by adapter (one gather launch): the step boundary.  A serving loop calls it once
+        per step; ``invoke_one_layer_*`` call it themselves when they are handed another index tensor than the one
+        the current plan was made from, or the same one after torch has written to it.  A tensor whose contents
+        were changed behind torch's back (a raw kernel writing through its pointer) needs this call."""
+        src = self._index_source(bsz, lora_ids)
+        cur_inds = self._indices(bsz, lora_ids, self.q_down.device)
         reuse = self._plan if (self._plan is not None and self._plan.T == bsz) else None
         self._plan = ops.plan_decode_ref(cur_inds, self.batch_size, self.n_layers, self.lora_rank, out=reuse)
-        self._plan_key = (cur_inds.data_ptr(), cur_inds._version, bsz)
+        self._plan_src, self._plan_ver = src, src._version
+        self._plan_gen += 1
         self._qkv_key = None
+        return self._plan
+
+    def _plan_for(self, bsz, lora_ids):
+        src = self._index_source(bsz, lora_ids)
+        if self._plan is None or self._plan_src is not src or self._plan_ver != src._version or self._plan.T != bsz:
+            self.plan_decode(bsz, lora_ids)
         return self._plan
 
     def invoke_one_layer_qkv(self, x, layer_id, lora_ids=None):
@@ -97,14 +112,12 @@ class Lora_GPU:
         bsz = x.shape[0]
         if not ops.ref_rank_supported(self.lora_rank):
             return tuple(self._invoke_single(n, x, layer_id, lora_ids) for n in "qkv")
-        cur_inds = self._indices(bsz, lora_ids, x.device)
-        if self._plan is None or self._plan_key != (cur_inds.data_ptr(), cur_inds._version, bsz):
-            self.plan_decode(bsz, cur_inds)
+        plan = self._plan_for(bsz, lora_ids)
         if not x.is_contiguous():
             x = x.contiguous()
         ys = [torch.empty(bsz, self.output_size, device=x.device, dtype=x.dtype) for _ in range(3)]
         ops.add_lora_bgmv_multi(ys, [x, x, x], [self.q_down, self.k_down, self.v_down], [self.q_up, self.k_up, self.v_up],
-                                self._plan, layer_id, 1.0, accumulate=False)
+                                plan, layer_id, 1.0, accumulate=False)
         return tuple(ys)
 
     def _invoke_single(self, name, x, layer_id, lora_ids):
@@ -130,13 +143,16 @@ class Lora_GPU:
             return self._invoke_single(name, x, layer_id, lora_ids)
         # ``_get_qkv`` asks for q, k and v of the same input one after the other
         # (transformer_layer_infer.py:109-111): the first of the three calls computes all of them in one call pair,
-        # the other two are answered from that result as long as the input tensor, its contents (torch's version
-        # counter), the layer and the index vector are the same.
-        cur_inds = self._indices(bsz, lora_ids, x.device)
-        key = (x.data_ptr(), x._version, tuple(x.shape), layer_id, cur_inds.data_ptr(), cur_inds._version)
-        if self._qkv_key != key or name not in self._qkv:
-            q, k, v = self.invoke_one_layer_qkv(x, layer_id, cur_inds)
-            self._qkv, self._qkv_key = {"q": q, "k": k, "v": v}, key
+        # the other two are answered from that result as long as it is the same input tensor object at the same
+        # torch version, the same layer, the same plan and the same weight tensors at the same versions.
+        self._plan_for(bsz, lora_ids)
+        weights = [getattr(self, f"{n}_{side}") for n in "qkv" for side in ("down", "up")]
+        key = (x._version, tuple(x.shape), layer_id, self._plan_gen, tuple(w._version for w in weights))
+        fresh = (self._qkv_key != key or self._qkv_x is not x or name not in self._qkv
+                 or any(a is not b for a, b in zip(self._qkv_w, weights)))
+        if fresh:
+            q, k, v = self.invoke_one_layer_qkv(x, layer_id, lora_ids)
+            self._qkv, self._qkv_x, self._qkv_w, self._qkv_key = {"q": q, "k": k, "v": v}, x, weights, key
         return self._qkv.pop(name)
 
     def invoke_one_layer_q(self, x, layer_id, prefill=False, lora_ids=None):

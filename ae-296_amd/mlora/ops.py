@@ -64,7 +64,20 @@ class DecodePlan:
         return self.tok_adapter.numel()
 
 
-N_CUS = 256       # compute units of the device the kernels are written for
+_n_cus = {}
+
+
+def n_cus(device=None) -> int:
+    """Compute units of `device` (default: the current one), asked once per device; where no device is present
+    (planning on a host without a GPU) the MI355X's 256."""
+    if not torch.cuda.is_available():
+        return 256
+    idx = torch.cuda.current_device() if device is None else torch.device(device).index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    if idx not in _n_cus:
+        _n_cus[idx] = int(torch.cuda.get_device_properties(idx).multi_processor_count)
+    return _n_cus[idx]
 
 
 def default_group(T: int) -> int:
@@ -84,7 +97,7 @@ def decode_fused(T: int, group: int, n_proj: int, n_slots: int) -> bool:
     if group > 2:
         return False
     items = T if group == 1 else (T + 1) // 2 + min(T, n_slots) // 2
-    return items * n_proj <= N_CUS
+    return items * n_proj <= n_cus()
 
 
 def group_for(T: int, n_proj: int, n_slots: int) -> int:

@@ -221,71 +221,3 @@ class TraceRunner:
             ops.bgmv(ys, [xl, xl, xl], self.pool, l, ["q", "k", "v"], tok, plan=plan, accumulate=accumulate)
         ev.record()
         return slots, self.y
-
-
-def bench_trace(args, dev, steps, warmup, n_adapters: int = 128, n_slots: int = 64):
-    """bench.py leg `maf_trace`: the decode steps of the reference's 512-arrival-rate trace (adapter ids from its
-    popularity vector of `n_adapters` adapters) on Llama-7B q/k/v shapes, rank 16, a pool of `n_slots` slots, eager
-    launches (the batch changes every step); reports decode steps per second and the per-layer call time."""
-    import os
-    import time
-
-    import torch
-
-    from . import workloads
-    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "..", "tests", "golden")
-    times = np.load(os.path.join(root, "maf_trace_512.npy"), allow_pickle=False)
-    pop = np.load(os.path.join(root, f"maf_popularity_{n_adapters}.npy"), allow_pickle=False)
-    ids = workloads.draw_lora_ids(pop, len(times), seed=0)
-    lens = draw_output_lengths(len(times), mean=256.0, seed=1)
-    sim = simulate(times, ids, lens, step_s=0.03, running_max_req_size=256, max_prefill_batch_size=8)
-    decode = [s for s in sim if s.kind == "decode" and len(s.lora_ids) > 0]
-    L, H, r = 32, 4096, 16
-    run = TraceRunner(L, H, r, n_slots, device=dev, max_batch=256)
-    n_steps = min(len(decode), max(steps, 200))
-    first = min(len(decode) - n_steps, 400)                  # past the ramp-up of the trace
-    window = decode[first:first + n_steps]
-    warm = decode[max(0, first - max(warmup, 20)):first]
-    # the adapters live in pinned host memory before the replay starts (drawing their weights is not part of a step)
-    for a in sorted({int(a) for s in warm + window for a in s.lora_ids}):
-        run.host[a] = run.loader.stage(run.adapter_weights(a), run.rank, run.scaling)
-    for s in warm:
-        run.decode_step(s.lora_ids)
-    torch.cuda.synchronize()
-    loads0 = run.residency.loads
-    per = []
-    t0 = time.perf_counter()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for s in window:
-        t1 = time.perf_counter()
-        run.decode_step(s.lora_ids)
-        per.append((time.perf_counter() - t1) * 1e3)
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    gpu_ms = e0.elapsed_time(e1)
-    sizes = np.array([len(s.lora_ids) for s in window])
-    touched = np.array([len(set(s.lora_ids.tolist())) for s in window])
-    tokproj = int(sizes.sum()) * 3 * L
-    s_per = sorted(per)
-    pick = lambda q: s_per[min(len(s_per) - 1, int(round(q * (len(s_per) - 1))))]
-    ms_per_step = wall * 1e3 / n_steps
-    # algorithmic bytes of the window: per step and layer, x once per projection, y read + written, touched adapters' rows once
-    alg = float(sum(3 * (t * H * 2 + 2 * t * H * 2 + u * r * 2 * H * 2 + 4 * t) for t, u in zip(sizes, touched))) * L
-    achieved = alg / (gpu_ms * 1e-3) / 1e9
-    return {"metric": "decode steps per second on the reference's arrival trace", "value": n_steps / wall, "unit": "steps/s",
-            "n_gpus": 1, "steps": n_steps, "warmup": warmup, "ms_per_step": ms_per_step,
-            "ms_per_step_spread": {"p10": pick(0.1), "p50": pick(0.5), "p90": pick(0.9)}, "higher_is_better": True,
-            "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-            "config": {"workload": f"maf_trace_512 arrivals, adapter per request from popularity_{n_adapters}, continuous batching "
-                                   f"(256 running, 8 admitted per step), Llama-7B q/k/v 4096->4096, rank 16, {n_slots}-slot paged pool, "
-                                   "32 layers, eager launches", "form": "gather + one BGMV call per layer, swap-in on miss",
-                       "steps_in_trace": len(decode), "tokens": float(sizes.mean()), "adapters_touched_per_step": float(touched.mean()),
-                       "swap_ins": run.residency.loads - loads0, "token_projections_per_s": tokproj / wall,
-                       "gpu_ms_per_step": gpu_ms / n_steps},
-            "roofline": {"bound": "hbm", "achieved": achieved, "peak": 8000.0, "unit": "GB/s", "frac": achieved / 8000.0,
-                         "traffic": None, "traffic_source": None,
-                         "kernel": "gather + 32 x BGMV call (q, k, v), batch changing every step, eager",
-                         "algorithmic_bytes_per_step": alg / n_steps},
-            "cpu_baseline": None}

@@ -143,8 +143,13 @@ def stream_ceiling(dev):
     is served by the last-level cache."""
     import torch
 
+    import ctypes
+
     import mlora
-    lib = mlora._ext.lib()
+    # the probe kernel lives in a library of its own beside the product one (built by the same Makefile)
+    probe = ctypes.CDLL(os.path.join(os.path.dirname(mlora._ext.LIB_PATH), "libmlora_probe.so"))
+    probe.mlora_probe_stream.restype = ctypes.c_int
+    probe.mlora_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_longlong, ctypes.c_int, ctypes.c_void_p]
     buf = torch.empty(3 << 30, dtype=torch.uint8, device=dev)
     buf.zero_()
     out = {}
@@ -155,7 +160,9 @@ def stream_ceiling(dev):
         def run():
             off = (state["i"] % n_regions) * nbytes
             state["i"] += 1
-            mlora._ext.check(lib.mlora_probe_stream(buf.data_ptr() + off, nbytes, mode, mlora._ext.current_stream_ptr()))
+            rc = probe.mlora_probe_stream(buf.data_ptr() + off, nbytes, mode, mlora._ext.current_stream_ptr())
+            if rc:
+                raise RuntimeError(f"mlora_probe_stream failed with {rc}")
 
         # launches back to back between two events (an event per launch would add its own gap to a 13 us launch);
         # best of five such blocks
@@ -256,6 +263,7 @@ def cpu_baseline(seconds=3.0):
     p1, pall = port(1), port(all_threads)
     t1, tall = torch_ref(1), torch_ref(all_threads)
     return {"value": pall["value"], "unit": "token-projections/s", "cores": all_threads, "kind": "port",
+            "workload": "config 1: single LoRA-delta op on the CPU reference path (not the headline's config 5)",
             "sample": f"config 1 (32 decode tokens, 8 rank-16 adapters, 4096->4096, fp32 weights, one task per token) repeated for "
                       f"{seconds:.0f} s per figure: libmlora_cpu.so on 1 and on {all_threads} persistent worker threads, torch "
                       f"(x.float() @ down @ up -> half per request) on 1 and on {all_threads} threads",
@@ -807,8 +815,12 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
                                      "kernels": "gather + prefill plan + 32 x (decode pair + SGMV shrink, reduce, expand over 7 projections)"}})
     traffic, src = traffic_of(workload, group == mlora.ops.group_for(cfg["T"], len(projs), cfg["N"]) and L == cfg["layers"] and not fused)
 
+    metric = "BGMV decode throughput (LoRA-applied token-projections per second)"
+    if pre is not None:
+        metric = (f"multi-LoRA apply throughput of the mixed step ({T} decode tokens through BGMV + {pre['T']} prefill tokens "
+                  "through SGMV, LoRA-applied token-projections per second)")
     out = {
-        "metric": "BGMV decode throughput (LoRA-applied token-projections per second)",
+        "metric": metric,
         "value": value, "unit": "token-projections/s", "n_gpus": 1, "steps": reps, "warmup": warmup,
         "ms_per_step": ms_per_step, "ms_per_step_spread": {k: t[k] for k in ("p10", "p50", "p90")},
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -818,7 +830,10 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
                    "form": "fused" if fused else "shrink + expand",
                    "tokens": T, "prefill_tokens": pre["T"] if pre else 0, "adapters": cfg["N"],
                    "adapters_touched": int(len(uniq)), "group": group,
-                   "hip_graph": not args.no_graph, "timed_region_ms": t["timed_ms"], "wall_s_timed_region": t["wall_s"]},
+                   "hip_graph": not args.no_graph, "timed_region_ms": t["timed_ms"], "wall_s_timed_region": t["wall_s"],
+                   # the decode half alone: the layers' BGMV calls without gather, plan and prefill launches
+                   "decode_only_token_projections_per_s": T * len(projs) * L / (tk["ms"] * 1e-3),
+                   "decode_only_ms_per_step": tk["ms"]},
         "roofline": dict({"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                           "frac": achieved / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": src, "kernel": kernel}, **extra),
         "cpu_baseline": None,
@@ -827,6 +842,74 @@ def bench_decode(args, dev, workload, steps, warmup, min_ms=0.0):
         te = timed(step, max(5, min(reps, 50)), 2)
         out["config"]["eager_ms_per_step"] = te["ms"]
     return out
+
+
+# ---------------------------------------------------------------------------------------------- arrival trace
+def bench_trace(args, dev, steps, warmup, n_adapters=128, n_slots=64):
+    """bench.py leg `maf_trace`: the decode steps of the reference's 512-arrival-rate trace (adapter ids from its
+    popularity vector of `n_adapters` adapters) on Llama-7B q/k/v shapes, rank 16, a pool of `n_slots` slots, eager
+    launches (the batch changes every step); reports decode steps per second and the per-layer call time."""
+    import numpy as np
+    import torch
+
+    from mlora import workloads
+    from mlora.trace_driver import TraceRunner, draw_output_lengths, simulate
+    root = os.path.join(ROOT, "tests", "golden")
+    times = np.load(os.path.join(root, "maf_trace_512.npy"), allow_pickle=False)
+    pop = np.load(os.path.join(root, f"maf_popularity_{n_adapters}.npy"), allow_pickle=False)
+    ids = workloads.draw_lora_ids(pop, len(times), seed=0)
+    lens = draw_output_lengths(len(times), mean=256.0, seed=1)
+    sim = simulate(times, ids, lens, step_s=0.03, running_max_req_size=256, max_prefill_batch_size=8)
+    decode = [s for s in sim if s.kind == "decode" and len(s.lora_ids) > 0]
+    L, H, r = 32, 4096, 16
+    run = TraceRunner(L, H, r, n_slots, device=dev, max_batch=256)
+    n_steps = min(len(decode), max(steps, 200))
+    first = min(len(decode) - n_steps, 400)                  # past the ramp-up of the trace
+    window = decode[first:first + n_steps]
+    warm = decode[max(0, first - max(warmup, 20)):first]
+    # the adapters live in pinned host memory before the replay starts (drawing their weights is not part of a step)
+    for a in sorted({int(a) for s in warm + window for a in s.lora_ids}):
+        run.host[a] = run.loader.stage(run.adapter_weights(a), run.rank, run.scaling)
+    for s in warm:
+        run.decode_step(s.lora_ids)
+    torch.cuda.synchronize()
+    loads0 = run.residency.loads
+    per = []
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for s in window:
+        t1 = time.perf_counter()
+        run.decode_step(s.lora_ids)
+        per.append((time.perf_counter() - t1) * 1e3)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_ms = e0.elapsed_time(e1)
+    sizes = np.array([len(s.lora_ids) for s in window])
+    touched = np.array([len(set(s.lora_ids.tolist())) for s in window])
+    tokproj = int(sizes.sum()) * 3 * L
+    s_per = sorted(per)
+    pick = lambda q: s_per[min(len(s_per) - 1, int(round(q * (len(s_per) - 1))))]
+    ms_per_step = wall * 1e3 / n_steps
+    # algorithmic bytes of the window: per step and layer, x once per projection, y read + written, touched adapters' rows once
+    alg = float(sum(3 * (t * H * 2 + 2 * t * H * 2 + u * r * 2 * H * 2 + 4 * t) for t, u in zip(sizes, touched))) * L
+    achieved = alg / (gpu_ms * 1e-3) / 1e9
+    return {"metric": "decode steps per second on the reference's arrival trace", "value": n_steps / wall, "unit": "steps/s",
+            "n_gpus": 1, "steps": n_steps, "warmup": warmup, "ms_per_step": ms_per_step,
+            "ms_per_step_spread": {"p10": pick(0.1), "p50": pick(0.5), "p90": pick(0.9)}, "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"maf_trace_512 arrivals, adapter per request from popularity_{n_adapters}, continuous batching "
+                                   f"(256 running, 8 admitted per step), Llama-7B q/k/v 4096->4096, rank 16, {n_slots}-slot paged pool, "
+                                   "32 layers, eager launches", "form": "gather + one BGMV call per layer, swap-in on miss",
+                       "steps_in_trace": len(decode), "tokens": float(sizes.mean()), "adapters_touched_per_step": float(touched.mean()),
+                       "swap_ins": run.residency.loads - loads0, "token_projections_per_s": tokproj / wall,
+                       "gpu_ms_per_step": gpu_ms / n_steps},
+            "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                         "traffic": None, "traffic_source": None,
+                         "kernel": "gather + 32 x BGMV call (q, k, v), batch changing every step, eager",
+                         "algorithmic_bytes_per_step": alg / n_steps},
+            "cpu_baseline": None}
 
 
 def leg_of(line):
@@ -901,8 +984,7 @@ def main():
         if workload == "reflayout":
             return bench_reflayout(args, dev, steps, warmup, min_ms)
         if workload == "maf_trace":
-            from mlora import trace_driver
-            return trace_driver.bench_trace(args, dev, steps, warmup)
+            return bench_trace(args, dev, steps, warmup)
         if workload == "swap":
             return bench_swap(args, dev)
         if workload == "assist":
@@ -934,12 +1016,40 @@ def main():
     log("headline: config 5 ...")
     line = bench_decode(args, dev, "c5", args.steps, args.warmup, 0.0)
     line["stream_ceiling"] = ceiling
-    line["legs"] = legs
     if not args.no_cpu:
         log("timing the CPU baseline ...")
         line["cpu_baseline"] = cpu_baseline()
-    line["config"]["bench_wall_s"] = time.perf_counter() - t_start
-    print(json.dumps(line), flush=True)
+    # The legs' figures as flat scalars of `config` (nested objects may be dropped by whoever stores the line):
+    # fraction of the HBM peak for every leg that is bound by it, MFMA figures for the prefill legs.
+    flat = line["config"]
+    flat["c5_decode_hbm_frac"] = line["roofline"]["frac"]
+    flat["c5_decode_launch_us"] = line["roofline"]["launch_us"]
+    flat["c5_whole_step_hbm_frac"] = line["roofline"]["whole_step"]["frac"]
+    for w, leg in legs.items():
+        if "error" in leg:
+            flat[f"{w}_error"] = leg["error"]
+            continue
+        rf = leg["roofline"]
+        flat[f"{w}_ms_per_step"] = leg["ms_per_step"]
+        if rf["bound"] == "hbm":
+            flat[f"{w}_hbm_frac"] = rf["frac"]
+        if "launch_us" in rf:
+            flat[f"{w}_launch_us"] = rf["launch_us"]
+        if w == "c4":
+            flat["c4_tflops"] = rf["mfma_tflops"]
+            flat["c4_mfma_frac"] = rf["mfma_frac"]
+            flat["c4_mfma_ceiling"] = rf["mfma_frac_ceiling"]
+        if w == "f1":
+            flat["f1_tflops"] = rf["achieved"]
+            flat["f1_mfma_frac"] = rf["frac"]
+        if w == "coldstart":
+            for k in ("cached_ms", "cpu_assisted_ms", "on_demand_ms", "ordering_holds"):
+                flat[f"coldstart_{k}"] = leg.get(k)
+    flat["bench_wall_s"] = time.perf_counter() - t_start
+    # key order of the printed line: the legs first, the headline's own fields (and the flat scalars) last
+    ordered = {"legs": legs}
+    ordered.update(line)
+    print(json.dumps(ordered), flush=True)
 
 
 if __name__ == "__main__":

@@ -124,14 +124,6 @@ int mlora_pool_scatter(int n_jobs, const void *const *src, void *const *dst_slab
                        int elt_bytes, void *stream);
 
 /*
- * Measurement helper, no counterpart in the reference: one plain streaming pass over `bytes` of device memory
- * (mode 0: read every 16 bytes once with nontemporal loads; mode 1: read, change and write back in place), so
- * that a benchmark can print what a memory-bound launch reaches on the device at hand beside the LoRA kernels'
- * figures.  Mode 1 adds 1 to the first 32-bit word of every 16 bytes.
- */
-int mlora_probe_stream(void *buf, int64_t bytes, int mode, void *stream);
-
-/*
  * CPU-assist transport: the GPU side of the path on which host workers compute the LoRA delta while an
  * adapter is still loading (HIP equivalents of the reference's tensor_cp copy family,
  * csrc/cuda_ops.hpp:109-229; no arithmetic here -- the workers are the reference's own processes or any
@@ -320,6 +312,13 @@ int mlora_sgmv_planned(void *y, const void *x, const void *a_rows, const void *b
  * Replaces the three torch.bmm pairs of lora_gpu.py:127-128,145-146,157-158 for one layer.
  */
 int64_t mlora_sgmv_multi_workspace_bytes(int T, int n_seg, int n_proj);
+/*
+ * Columns of y that one expand workgroup of such a call covers for a projection of width hout (the library
+ * picks 512, or the width whose block count per 64-token tile suits the order its workgroups run in: 640 for
+ * hout 5120, 576 for 13824).  Informational, like the workspace sizes; 0 for arguments out of range.  No
+ * counterpart in the reference (its prefill is two library GEMMs, lora_gpu.py:127-128).
+ */
+int mlora_sgmv_expand_cols(int T, int n_seg, int n_proj, int hout);
 int mlora_sgmv_multi_planned(int n_proj, void *const *y, const void *const *x,
                              const void *const *a_rows, const void *const *b_rows,
                              const int32_t *hin, const int32_t *hout,

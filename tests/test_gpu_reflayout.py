@@ -111,10 +111,10 @@ def test_lora_gpu_qkv_in_one_call_pair_and_served_to_the_three_calls():
         want = torch.stack([x[i].float() @ down[ids[i], 2].float().t() @ up[ids[i], 2].float().t() for i in range(bsz)])
         assert got.shape == (bsz, 512) and torch.allclose(got.float(), want, rtol=RTOL, atol=ATOL)
     q1 = g.invoke_one_layer_q(x, 2, False, lora_ids=ids)
-    plan_after_q = g._plan_key
+    plan_after_q = g._plan_gen
     k1 = g.invoke_one_layer_k(x, 2, False, lora_ids=ids)
     v1 = g.invoke_one_layer_v(x, 2, False, lora_ids=ids)
-    assert g._plan_key == plan_after_q                        # one plan, made before
+    assert g._plan_gen == plan_after_q                        # one plan, made before
     assert torch.equal(q1, q) and torch.equal(k1, k) and torch.equal(v1, v)
     x.mul_(2.0)                                                # same storage, new contents
     q2 = g.invoke_one_layer_q(x, 2, False, lora_ids=ids)
@@ -123,6 +123,44 @@ def test_lora_gpu_qkv_in_one_call_pair_and_served_to_the_three_calls():
     k2 = g.invoke_one_layer_k(x, 2, False, lora_ids=ids)
     want = torch.stack([x[i].float() @ g.k_down[ids[i], 2].float().t() @ g.k_up[ids[i], 2].float().t() for i in range(bsz)])
     assert torch.allclose(k2.float(), want, rtol=RTOL, atol=ATOL)
+
+
+def test_lora_gpu_fresh_index_tensor_every_step():
+    """A serving loop builds lora_ids afresh each step (pre_process.py:50,100); a freed tensor's address is handed to
+    the next one of the same size.  Every step must be computed from its own ids; in-place edits through torch and
+    weight writes are seen as well."""
+    cfg = dict(n_layers=2, batch_size=16, lora_rank=16, hidden_dim=512, tp_degree=1, max_prefill_batch_size=2)
+    g = Lora_GPU(cfg, seed=9)
+    bsz = 13
+    x = torch.randn(bsz, 512, device="cuda", dtype=torch.float16)
+
+    def want_of(name, ids, layer):
+        down, up = getattr(g, f"{name}_down"), getattr(g, f"{name}_up")
+        return torch.stack([x[i].float() @ down[ids[i], layer].float().t() @ up[ids[i], layer].float().t() for i in range(bsz)])
+
+    rng = np.random.default_rng(21)
+    addresses = set()
+    say("Lora_GPU: fresh int32 lora_ids per step")
+    for step in range(6):
+        host = rng.integers(0, 16, bsz).tolist()
+        ids = torch.tensor(host, dtype=torch.int32, device="cuda")     # as pre_process.py:100 makes them
+        addresses.add(ids.data_ptr())
+        for layer in range(2):
+            for name in "qkv":
+                got = getattr(g, f"invoke_one_layer_{name}")(x, layer, False, lora_ids=ids)
+                assert torch.allclose(got.float(), want_of(name, host, layer), rtol=RTOL, atol=ATOL), (step, layer, name)
+        del ids                                                         # the next step's tensor may reuse the address
+    assert len(addresses) < 6, "the allocator never reused an address: the case this test is about did not occur"
+    # the same tensor object edited in place through torch
+    ids = torch.tensor(rng.integers(0, 16, bsz).tolist(), dtype=torch.int32, device="cuda")
+    g.invoke_one_layer_q(x, 0, False, lora_ids=ids)
+    ids.copy_(torch.tensor(host, dtype=torch.int32, device="cuda"))
+    got = g.invoke_one_layer_q(x, 0, False, lora_ids=ids)
+    assert torch.allclose(got.float(), want_of("q", host, 0), rtol=RTOL, atol=ATOL)
+    # weights written in place between the q call and the k call of one layer
+    g.k_down[host[0], 0].mul_(-3.0)
+    got = g.invoke_one_layer_k(x, 0, False, lora_ids=ids)
+    assert torch.allclose(got.float(), want_of("k", host, 0), rtol=RTOL, atol=ATOL)
 
 
 def test_add_lora_bgmv_bad_index_leaves_row_untouched():
