@@ -85,8 +85,7 @@ __device__ __forceinline__ int slice_factor(int r)
 // Shrink of one (item, projection, column slice) over the first 4 * NR rank rows (NR per 16-lane
 // row).  The caller picks the smallest NR that covers the item's rank, so an adapter of rank 8 in a
 // pool that goes up to rank 64 issues loads for 8 rows, not 64.
-// COH: the sums are stored for readers on other compute units of the same launch (agent-scope stores).
-template <int DT, int G, int RMAX, int KSC, int NR, bool HOT, bool COH = false, class RowsPtr>
+template <int DT, int G, int RMAX, int KSC, int NR, bool HOT, class RowsPtr>
 __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, RowsPtr rows, const int (&tok)[G],
                                             int r, int proj, int ks, int slot, float (&s_part)[4][G][RMAX])
 {
@@ -188,9 +187,7 @@ __device__ __forceinline__ void shrink_rows(const BgmvArgs &p, RowsPtr rows, con
             float s = 0.f;
 #pragma unroll
             for (int wv = 0; wv < NW; wv++) s += s_part[wv][k][j];
-            float *dst = p.vws + (((size_t)proj * p.T + tok[k]) * p.ks_max + slot) * RMAX + j;
-            if constexpr (COH) __hip_atomic_store(dst, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            else *dst = s;
+            p.vws[(((size_t)proj * p.T + tok[k]) * p.ks_max + slot) * RMAX + j] = s;
         }
     }
 }
@@ -546,451 +543,6 @@ __global__ __launch_bounds__(256) void bgmv_expand_bt_kernel(const BgmvArgs p)
     } while (false);
 }
 
-// ---------------------------------------------------------------------------------------------------------------
-// One launch for calls of about one round of workgroups ("chained" form).
-//
-// The grid holds the shrink units first and the expand units after them.  Workgroups are dispatched in id order,
-// so every shrink unit is on a compute unit (or done) before the first expand unit starts; an expand unit requests
-// its B rows and its y rows right away and only then waits for the shrink units of its (record, projection), so
-// the second launch's start-up (a dependent launch, record and row-index loads, the first rows' latency) runs
-// under the tail of the shrink instead of after it.
-//
-// Units are sized by rank bucket so that each moves about the same number of row bytes (16 row loads of 16 bytes
-// per lane): an item of more than 32 rank rows is cut into 512-column units, 17..32 rows into 1024-column units,
-// up to 16 rows into 2048-column units.  The trailer record of the plan says how many items each bucket holds
-// (the list is ordered by bucket), so unit u maps to (item, projection, slice) by arithmetic and the grid holds
-// no workgroups for slices an item does not have.  A workgroup takes units u, u + grid, ... (one for most calls).
-//
-// Hand-over of the sums: a shrink unit stores them with agent-scope stores, waits for the stores to complete and
-// adds 1 to its (record, projection)'s counter: words 12..15 of the record, 16 bits per projection, the low byte
-// counting shrink units that have arrived and the high byte expand units that have finished.  An expand unit polls
-// the counter (bounded: after `spin_limit` polls it computes the sums itself from x and A, so every workgroup
-// ends whatever the order of dispatch), reads the sums with agent-scope loads, and when done adds 0x100; whoever
-// brings the field to its full count takes the count off again, so the records are left as the gather wrote them.
-// Calls that use the same records must therefore be ordered on one stream.
-template <int RMAX> struct ChainGeom;
-// shrink: 16-byte chunks per unit, by bucket (a launch never sees a bucket above its rank stride: clamped)
-template <> struct ChainGeom<64> { static constexpr int KSC0 = 64, KSC1 = 128, KSC2 = 256, KSC3 = 256, MINB = 0; };
-template <> struct ChainGeom<32> { static constexpr int KSC0 = 128, KSC1 = 128, KSC2 = 256, KSC3 = 256, MINB = 1; };
-template <> struct ChainGeom<16> { static constexpr int KSC0 = 256, KSC1 = 256, KSC2 = 256, KSC3 = 256, MINB = 2; };
-template <int RMAX> constexpr int chain_ksc(int bucket)
-{
-    using CG = ChainGeom<RMAX>;
-    return bucket == 0 ? CG::KSC0 : (bucket == 1 ? CG::KSC1 : (bucket == 2 ? CG::KSC2 : CG::KSC3));
-}
-// expand: columns per unit, by bucket
-__host__ __device__ constexpr int chain_cols(int bucket) { return bucket == 0 ? 512 : (bucket == 1 ? 1024 : 2048); }
-
-// Unit u of a part -> (bucket, position in the list, projection, slice); false beyond the last unit.
-__device__ __forceinline__ bool chain_unit(const int (&end)[WORK_BUCKETS][MAX_PROJ], int n_proj, const int (&nb)[WORK_BUCKETS],
-                                           int u, int &bucket, int &pos, int &proj, int &slice)
-{
-    int first = 0;
-#pragma unroll
-    for (int k = 0; k < WORK_BUCKETS; k++) {
-        const int per = end[k][n_proj - 1];
-        const int n = nb[k] * per;
-        if (u < n) {
-            const int i = u / per, q = u - i * per;
-            bucket = k; pos = first + i;
-            proj = 0;
-            while (proj + 1 < n_proj && q >= end[k][proj]) proj++;
-            slice = q - (proj ? end[k][proj - 1] : 0);
-            return true;
-        }
-        u -= n; first += nb[k];
-    }
-    return false;
-}
-
-// Counter field of (record, projection): 16 bits of words 12..15.
-__device__ __forceinline__ unsigned *chain_counter(const int32_t *rec, int proj, int &shift)
-{
-    shift = (proj & 1) * 16;
-    return reinterpret_cast<unsigned *>(const_cast<int32_t *>(rec)) + 12 + (proj >> 1);
-}
-
-// Adds `inc` to the field; the arrival that completes `full` (shrink units | expand units << 8) clears the field.
-__device__ __forceinline__ void chain_arrive(const int32_t *rec, int proj, unsigned inc, unsigned full)
-{
-    int shift;
-    unsigned *cw = chain_counter(rec, proj, shift);
-    const unsigned old = __hip_atomic_fetch_add(cw, inc << shift, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (((old >> shift) & 0xffffu) + inc == full)
-        __hip_atomic_fetch_sub(cw, full << shift, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-template <int DT, int G, int RMAX, int BK>
-__device__ __forceinline__ void chain_shrink_unit(const BgmvArgs &p, const int32_t *__restrict__ rec, int proj, int slice,
-                                                  unsigned full, float (&s_part)[4][G][RMAX])
-{
-    constexpr int MB = BK < ChainGeom<RMAX>::MINB ? ChainGeom<RMAX>::MINB : BK;   // geometry of the clamped bucket
-    constexpr int KSC = chain_ksc<RMAX>(MB);
-    constexpr int F = KSC / chain_ksc<RMAX>(ChainGeom<RMAX>::MINB);       // base slices per unit
-    constexpr int NR = MB == 0 ? 16 : (MB == 1 ? 8 : (MB == 2 ? 4 : 2));  // rank rows per 16-lane row
-    int ntok = rec[0];
-    if (ntok <= 0) return;
-    ntok = ntok < G ? ntok : G;
-    if (rec[1] < 0) return;                                     // no adapter: the expand side does not wait either
-    int r = rec[2];
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    int tok[G];
-#pragma unroll
-    for (int k = 0; k < G; k++) {
-        const int t = k < ntok ? rec[4 + k] : -1;
-        tok[k] = (t >= 0 && t < p.T) ? t : -1;
-    }
-    shrink_rows<DT, G, RMAX, KSC, NR, false, true>(p, rec + WORK_ROWS_AT, tok, r, proj, slice, slice * F, s_part);
-    // the sums are at the agent's coherence point before the counter says so
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (threadIdx.x == 0) chain_arrive(rec, proj, 1u, full);
-}
-
-template <int DT, int G, int RMAX, int BK>
-__device__ __forceinline__ void chain_expand_unit(const BgmvArgs &p, const int32_t *rec_rw, int proj, int slice,
-                                                  unsigned need_sh, unsigned full, float (&s_v)[G][RMAX], float *s_o, int *s_flag)
-{
-    constexpr int MB = BK < ChainGeom<RMAX>::MINB ? ChainGeom<RMAX>::MINB : BK;   // geometry of the clamped bucket
-    constexpr int C = chain_cols(MB);                           // columns per unit
-    constexpr int RG = MB == 0 ? 4 : (MB == 1 ? 2 : 1);         // rank groups (256 threads = RG x C / 8)
-    constexpr int RPG = MB == 3 ? 8 : 16;                       // rank rows per group = row loads in flight per lane
-    constexpr int CCH = C / 8;                                  // 16-byte column chunks per unit (a multiple of 64)
-    constexpr int NY = RG == 1 ? G : (G * CCH + 255) / 256;     // y chunks per thread in the final step
-    constexpr int KSTEP = chain_ksc<RMAX>(MB) / chain_ksc<RMAX>(ChainGeom<RMAX>::MINB);   // the shrink filled every KSTEP-th slot
-    static_assert(CCH % 64 == 0, "a wavefront belongs to one rank group");
-
-    const const_i32_ptr rec = as_const(rec_rw);                 // header and rows: scalar loads
-    const int tid = threadIdx.x;
-    const int grp = __builtin_amdgcn_readfirstlane(tid / CCH);  // uniform over the wavefront
-    const int cc = tid - grp * CCH;
-    const int hout = p.hout[proj], hin = p.hin[proj];
-    const int ncc_out = hout >> 3;
-    const int ch0 = slice * CCH;
-    const bool active = ch0 + cc < ncc_out;
-    char *__restrict__ y = static_cast<char *>(p.y[proj]);
-    const char *__restrict__ brows = static_cast<const char *>(p.b_rows[proj]);
-    const size_t row_bytes = (size_t)hout * 2u;
-
-    int ntok = rec[0];
-    if (ntok <= 0) return;
-    ntok = ntok < G ? ntok : G;
-    const int adapter = rec[1];
-    int r = rec[2];
-    r = r < 0 ? 0 : (r > RMAX ? RMAX : r);
-    const float scale = __builtin_bit_cast(float, rec[3]);
-    int tok[G];
-#pragma unroll
-    for (int k = 0; k < G; k++) {
-        const int t = k < ntok ? rec[4 + k] : -1;
-        tok[k] = (t >= 0 && t < p.T) ? t : -1;
-    }
-
-    // Which (token, column chunk) pairs this thread reads, updates and writes in the final step.  Loads are issued
-    // for every pair at a clamped address (token 0, last chunk) and only the stores are conditional: a load under
-    // a per-lane condition costs a branch and registers carried around it.
-    int ytok[NY];
-    unsigned yoff[NY];                                          // byte offset of the chunk inside its row
-    bool ylive[NY];
-#pragma unroll
-    for (int m = 0; m < NY; m++) {
-        int c;
-        if constexpr (RG == 1) { ytok[m] = tok[m]; c = cc; ylive[m] = tok[m] >= 0 && active; }
-        else {
-            const int e = tid + m * 256;
-            const int k = e / CCH;
-            c = e - k * CCH;
-            int t = -1;
-#pragma unroll
-            for (int kk = 0; kk < G; kk++) t = k == kk ? tok[kk] : t;
-            ytok[m] = t;
-            ylive[m] = t >= 0 && ch0 + c < ncc_out;
-        }
-        const int ch = ch0 + c < ncc_out ? ch0 + c : ncc_out - 1;
-        yoff[m] = (unsigned)ch * 16u;
-    }
-
-    if (adapter < 0) {
-        if (!p.accumulate) {
-#pragma unroll
-            for (int m = 0; m < NY; m++)
-                if (ylive[m]) stg16(y + (size_t)ytok[m] * row_bytes + yoff[m], zero16());
-        }
-        return;
-    }
-
-    // everything that does not depend on the shrink is requested before the wait: a rank row's address is the same
-    // for the whole wavefront (scalar registers), a lane adds its column offset; an absent row (a uniform condition)
-    // is not read
-    const unsigned voff = (unsigned)(active ? ch0 + cc : ncc_out - 1) * 16u;
-    auto load_b = [&](uint4 (&bv)[RPG]) {
-#pragma unroll
-        for (int i = 0; i < RPG; i++) {
-            const int j = grp * RPG + i;
-            int row = rec[WORK_ROWS_AT + j];
-            const bool ok = j < r && row >= 0 && row < p.pool.n_rows_b;      // uniform over the wavefront: a scalar branch
-            if (ok) bv[i] = ldg16_stream(brows + (size_t)row * row_bytes + voff);
-            else bv[i] = zero16();
-        }
-    };
-    auto load_y = [&](uint4 (&yv)[NY]) {
-        if (p.accumulate) {
-#pragma unroll
-            for (int m = 0; m < NY; m++) yv[m] = ldg16_stream(y + (size_t)(ytok[m] >= 0 ? ytok[m] : 0) * row_bytes + yoff[m]);
-        } else {
-#pragma unroll
-            for (int m = 0; m < NY; m++) yv[m] = zero16();
-        }
-    };
-    uint4 bv[RPG];
-    uint4 yv[NY];
-    load_b(bv);
-    load_y(yv);
-
-    // bounded wait for the shrink units of this (record, projection)
-    if (tid == 0) {
-        int shift;
-        unsigned *cw = chain_counter(rec_rw, proj, shift);
-        int ok = 0;
-        for (int spin = 0; spin < p.chain.spin_limit; spin++) {
-            if (((__hip_atomic_load(cw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >> shift) & 0xffu) >= need_sh) { ok = 1; break; }
-            __builtin_amdgcn_s_sleep(2);
-        }
-        *s_flag = ok;
-    }
-    __syncthreads();
-    const bool arrived = *s_flag != 0;
-
-    if (arrived) {
-        // v = scaling * (sum of the slices' partial sums), slices added in ascending order, twelve requested at a time
-        const int n_ks = ((hin >> 3) + chain_ksc<RMAX>(ChainGeom<RMAX>::MINB) - 1) / chain_ksc<RMAX>(ChainGeom<RMAX>::MINB);
-        for (int e = tid; e < G * RMAX; e += 256) {
-            const int k = e / RMAX, j = e - k * RMAX;
-            int t = -1;
-#pragma unroll
-            for (int kk = 0; kk < G; kk++) t = k == kk ? tok[kk] : t;
-            float s = 0.f;
-            if (j < r && t >= 0) {
-                const float *src = p.vws + (((size_t)proj * p.T + t) * p.ks_max) * RMAX + j;
-                for (int ks0 = 0; ks0 < n_ks; ks0 += 12 * KSTEP) {
-                    float q[12];
-#pragma unroll
-                    for (int u = 0; u < 12; u++) {
-                        const int ks = ks0 + u * KSTEP;
-                        q[u] = ks < n_ks ? __hip_atomic_load(src + (size_t)ks * RMAX, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 12; u++) s += q[u];
-                }
-            }
-            s_v[k][j] = s * scale;
-        }
-    } else {
-        // The shrink units have not shown up within the limit: the sums are computed here, one (token, rank row) at a
-        // time over the whole row.  Slow and never taken under in-order dispatch; it is what makes the wait bounded.
-        const uint16_t *__restrict__ arows = static_cast<const uint16_t *>(p.a_rows[proj]);
-        const uint16_t *__restrict__ x = static_cast<const uint16_t *>(p.x[proj]);
-        const int ncc_in = hin >> 3;
-        float *s_red = s_o;                                      // 4 floats
-#pragma unroll 1
-        for (int k = 0; k < G; k++) {
-            int t = -1;
-#pragma unroll
-            for (int kk = 0; kk < G; kk++) t = k == kk ? tok[kk] : t;
-#pragma unroll 1
-            for (int j = 0; j < RMAX; j++) {
-                const int row = j < r ? rec[WORK_ROWS_AT + j] : -1;
-                const bool ok = t >= 0 && row >= 0 && row < p.pool.n_rows_a;    // uniform over the workgroup
-                float acc = 0.f;
-                if (ok) {
-                    const uint4 *ap = reinterpret_cast<const uint4 *>(arows + (size_t)row * hin);
-                    const uint4 *xp = reinterpret_cast<const uint4 *>(x + (size_t)t * hin);
-#pragma unroll 1
-                    for (int c = tid; c < ncc_in; c += 256) acc = dot8<DT>(ldg16(ap + c), ldg16(xp + c), acc);
-                    acc = wave_sum(acc);
-                }
-                __syncthreads();                                 // s_red of the previous round has been read
-                if ((tid & 63) == 0) s_red[tid >> 6] = acc;
-                __syncthreads();
-                if (tid == 0) s_v[k][j] = (s_red[0] + s_red[1] + s_red[2] + s_red[3]) * scale;
-            }
-        }
-        load_b(bv);                                              // not kept across the slow path: requested again
-        load_y(yv);
-    }
-    __syncthreads();
-
-    // Lane k * RPG + i of every wavefront fetches v[k][first row of the group + i] once; the multiply-adds below take it
-    // from there as a scalar (v_readlane), so the inner loop holds no LDS reads and no copy of v per lane.
-    static_assert(G * RPG <= 64, "one value of v per lane");
-    const int vl = tid & 63;
-    float myv = vl < G * RPG ? s_v[vl / RPG][grp * RPG + vl % RPG] : 0.f;
-    float o[G][8];
-#pragma unroll
-    for (int k = 0; k < G; k++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[k][e] = 0.f;
-#pragma unroll
-    for (int i = 0; i < RPG; i++) {
-        float f[8];
-        unpack8<DT>(bv[i], f);
-#pragma unroll
-        for (int k = 0; k < G; k++) {
-            const float vk = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, myv), k * RPG + i));
-#pragma unroll
-            for (int e = 0; e < 8; e++) o[k][e] = fmaf(vk, f[e], o[k][e]);
-        }
-        // One row at a time: left alone, the compiler converts every row to fp32 and reads every v up front (eight
-        // registers per row).  Empty statements that name the sums, the next row and v keep each row's work behind
-        // the previous row's.
-#pragma unroll
-        for (int k = 0; k < G; k++)
-            asm volatile("" : "+v"(o[k][0]), "+v"(o[k][1]), "+v"(o[k][2]), "+v"(o[k][3]), "+v"(o[k][4]), "+v"(o[k][5]), "+v"(o[k][6]), "+v"(o[k][7]));
-        if (i + 1 < RPG) asm volatile("" : "+v"(bv[i + 1 < RPG ? i + 1 : i].x), "+v"(bv[i + 1 < RPG ? i + 1 : i].y), "+v"(bv[i + 1 < RPG ? i + 1 : i].z), "+v"(bv[i + 1 < RPG ? i + 1 : i].w), "+v"(myv));
-    }
-
-    if constexpr (RG == 1) {
-#pragma unroll
-        for (int k = 0; k < G; k++) {
-            float yf[8];
-            unpack8<DT>(yv[k], yf);                              // zeros when not accumulating
-#pragma unroll
-            for (int e = 0; e < 8; e++) yf[e] += o[k][e];
-            if (ylive[k]) stg16_stream(y + (size_t)ytok[k] * row_bytes + yoff[k], pack8<DT>(yf));
-        }
-    } else {
-        // the rank groups' partial results meet in LDS: s_o[group][token][column]
-#pragma unroll
-        for (int k = 0; k < G; k++) {
-            float4_t *dst = reinterpret_cast<float4_t *>(s_o + ((size_t)(grp * G + k) * C + cc * 8));
-            dst[0] = float4_t{o[k][0], o[k][1], o[k][2], o[k][3]};
-            dst[1] = float4_t{o[k][4], o[k][5], o[k][6], o[k][7]};
-        }
-        __syncthreads();
-#pragma unroll
-        for (int m = 0; m < NY; m++) {
-            const int e = tid + m * 256;
-            const int k = e / CCH, c = e - k * CCH;
-            float yf[8];
-            unpack8<DT>(yv[m], yf);
-            // rank groups added in ascending order and then on top of y: the same order whatever the token's place in the item
-            float d[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-            if (k < G) {
-#pragma unroll
-                for (int gq = 0; gq < RG; gq++) {
-                    const float4_t *src = reinterpret_cast<const float4_t *>(s_o + ((size_t)(gq * G + k) * C + c * 8));
-                    const float4_t a0 = src[0], a1 = src[1];
-                    d[0] += a0[0]; d[1] += a0[1]; d[2] += a0[2]; d[3] += a0[3];
-                    d[4] += a1[0]; d[5] += a1[1]; d[6] += a1[2]; d[7] += a1[3];
-                }
-            }
-#pragma unroll
-            for (int q = 0; q < 8; q++) yf[q] += d[q];
-            if (ylive[m]) stg16_stream(y + (size_t)ytok[m] * row_bytes + yoff[m], pack8<DT>(yf));
-        }
-    }
-    if (tid == 0) chain_arrive(rec_rw, proj, 0x100u, full);
-}
-
-template <int DT, int G, int RMAX>
-__global__ __launch_bounds__(256) void bgmv_chain_kernel(const BgmvArgs p)
-{
-    // LDS of the two parts overlaps: a workgroup is either a shrink or an expand workgroup
-    constexpr int SO_FLOATS = RMAX >= 32 ? 4 * G * 512 : 4;      // rank-group partials of a 512- or 1024-column unit
-    __shared__ __attribute__((aligned(16))) float s_o[SO_FLOATS > 4 * G * RMAX ? SO_FLOATS : 4 * G * RMAX];
-    __shared__ __attribute__((aligned(16))) float s_v[G][RMAX];
-    __shared__ int s_flag;
-    float (&s_part)[4][G][RMAX] = *reinterpret_cast<float (*)[4][G][RMAX]>(&s_o[0]);
-
-    const int32_t *__restrict__ tr = p.work + (size_t)(p.work_cap - 1) * WORK_WORDS + WORK_ROWS_AT;
-    const int n_chunks = tr[0];
-    const int nb[WORK_BUCKETS] = {tr[1], tr[2], tr[3], tr[4]};
-    if (n_chunks <= 0) return;
-    const int per_xcd = (n_chunks + 7) >> 3;
-    const bool is_sh = (int)blockIdx.x < p.chain.grid_sh;
-
-#ifdef ONLY_EX
-    if (false) {
-#else
-    if (is_sh) {
-#endif
-        for (int u = blockIdx.x;; u += p.chain.grid_sh) {
-            int bucket, pos, proj, slice;
-            if (!chain_unit(p.chain.sh_end, p.n_proj, nb, u, bucket, pos, proj, slice)) break;
-            const int b = (pos % per_xcd) * 8 + pos / per_xcd;
-            const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
-            const unsigned n_sh = (unsigned)(p.chain.sh_end[bucket][proj] - (proj ? p.chain.sh_end[bucket][proj - 1] : 0));
-            const unsigned n_ex = (unsigned)(p.chain.ex_end[bucket][proj] - (proj ? p.chain.ex_end[bucket][proj - 1] : 0));
-            const unsigned full = n_sh | (n_ex << 8);
-            if (bucket == 0) chain_shrink_unit<DT, G, RMAX, 0>(p, rec, proj, slice, full, s_part);
-            else if (bucket == 1) chain_shrink_unit<DT, G, RMAX, 1>(p, rec, proj, slice, full, s_part);
-            else if (bucket == 2) chain_shrink_unit<DT, G, RMAX, 2>(p, rec, proj, slice, full, s_part);
-            else chain_shrink_unit<DT, G, RMAX, 3>(p, rec, proj, slice, full, s_part);
-            __syncthreads();                                    // s_part is reused by the next unit
-        }
-    } else {
-#ifdef ONLY_SH
-        return;
-#endif
-        for (int u = blockIdx.x - p.chain.grid_sh;; u += p.chain.grid_ex) {
-            int bucket, pos, proj, slice;
-            if (!chain_unit(p.chain.ex_end, p.n_proj, nb, u, bucket, pos, proj, slice)) break;
-            const int b = (pos % per_xcd) * 8 + pos / per_xcd;
-            const int32_t *__restrict__ rec = p.work + (size_t)b * WORK_WORDS;
-            const unsigned n_sh = (unsigned)(p.chain.sh_end[bucket][proj] - (proj ? p.chain.sh_end[bucket][proj - 1] : 0));
-            const unsigned n_ex = (unsigned)(p.chain.ex_end[bucket][proj] - (proj ? p.chain.ex_end[bucket][proj - 1] : 0));
-            const unsigned full = n_sh | (n_ex << 8);
-            if (bucket == 0) chain_expand_unit<DT, G, RMAX, 0>(p, rec, proj, slice, n_sh, full, s_v, s_o, &s_flag);
-            else if (bucket == 1) chain_expand_unit<DT, G, RMAX, 1>(p, rec, proj, slice, n_sh, full, s_v, s_o, &s_flag);
-            else if (bucket == 2) chain_expand_unit<DT, G, RMAX, 2>(p, rec, proj, slice, n_sh, full, s_v, s_o, &s_flag);
-            else chain_expand_unit<DT, G, RMAX, 3>(p, rec, proj, slice, n_sh, full, s_v, s_o, &s_flag);
-            __syncthreads();                                    // s_v, s_o and s_flag are reused by the next unit
-        }
-    }
-}
-
-// Host side of the chained form: units per (bucket, projection) and the grid.
-template <int RMAX>
-static void chain_geometry(BgmvArgs &a)
-{
-    const DecodeOptions &opt = decode_options();
-    long long per_sh = 0, per_ex = 0;
-    for (int k = 0; k < WORK_BUCKETS; k++) {
-        const int mb = k < ChainGeom<RMAX>::MINB ? ChainGeom<RMAX>::MINB : k;
-        const int ksc = chain_ksc<RMAX>(mb), cols = chain_cols(mb);
-        int sh = 0, ex = 0;
-        for (int q = 0; q < MAX_PROJ; q++) {
-            if (q < a.n_proj) {
-                sh += ((a.hin[q] >> 3) + ksc - 1) / ksc;
-                ex += (a.hout[q] + cols - 1) / cols;
-            }
-            a.chain.sh_end[k][q] = sh; a.chain.ex_end[k][q] = ex;
-        }
-        per_sh = sh > per_sh ? sh : per_sh;
-        per_ex = ex > per_ex ? ex : per_ex;
-    }
-    const long long cap = opt.grid_cap > 0 ? opt.grid_cap : 1;
-    const long long n_sh = per_sh * a.items_cap, n_ex = per_ex * a.items_cap;
-    a.chain.grid_sh = (int)(n_sh < cap ? n_sh : cap);
-    a.chain.grid_ex = (int)(n_ex < cap ? n_ex : cap);
-    a.chain.spin_limit = opt.spin_limit;
-}
-
-template <int DT, int G, int RMAX>
-static int launch_chain(const BgmvArgs &a0, hipStream_t s)
-{
-    BgmvArgs a = a0;
-    chain_geometry<RMAX>(a);
-    if (a.chain.grid_sh <= 0 || a.chain.grid_ex <= 0) return 0;
-    // the sums are laid out by the base slice of the launch's rank stride
-    constexpr int base = chain_ksc<RMAX>(ChainGeom<RMAX>::MINB);
-    int ks_max = 0;
-    for (int q = 0; q < a.n_proj; q++) { const int n = ((a.hin[q] >> 3) + base - 1) / base; ks_max = n > ks_max ? n : ks_max; }
-    a.ks_max = ks_max;
-    hipLaunchKernelGGL((bgmv_chain_kernel<DT, G, RMAX>), dim3((unsigned)(a.chain.grid_sh + a.chain.grid_ex)), dim3(256), 0, s, a);
-    return (int)hipGetLastError();
-}
-
 // Records a launch covers (a multiple of 8, one per XCD residue): every workgroup walks records b, b + stride, ...
 // The host only knows an upper bound on the records in use (items_cap: T/G full pieces plus one short piece per
 // adapter present); a grid over the whole bound spends about a nanosecond per workgroup of an empty record on
@@ -1075,10 +627,6 @@ static int launch_sliced(const BgmvArgs &a, hipStream_t s)
     // compute unit): from about sixteen on, the items of a much-used adapter no longer run side by side.
     const long long rounds = (long long)a.sh_end[a.n_proj - 1] * a.items_cap / (3 * device_compute_units());
     if (rounds >= 16) return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, true>(a, s);
-    // about one round: the one-launch form, for plans whose list is ordered by rank bucket (at most 2048 tokens)
-    if constexpr (G <= 4) {
-        if (decode_options().chain && a.T <= 2048 && a.chain_ok) return launch_chain<DT, G, RMAX>(a, s);
-    }
     return launch_pair<DT, G, RMAX, Slices<RMAX>::KSC, Slices<RMAX>::NTE, false>(a, s);
 }
 void bgmv_split_slices(int max_rank, int *ksc, int *nte, bool transposed_b)
@@ -1111,21 +659,6 @@ static int launch_split_dt(const BgmvArgs &a, int group, int max_rank, hipStream
 }
 
 int bgmv_split_rank_stride(int max_rank) { return max_rank <= 16 ? 16 : (max_rank <= 32 ? 32 : 64); }
-
-DecodeOptions &decode_options()
-{
-    static DecodeOptions opt = {1, 1 << 20, 2048};
-    return opt;
-}
-
-// 16-byte chunks of the narrowest shrink slice any launch form uses at this rank stride (sizes the intermediate).
-int bgmv_min_slice_chunks(int max_rank)
-{
-    int ksc, nte;
-    bgmv_split_slices(max_rank, &ksc, &nte);
-    const int c = max_rank <= 16 ? chain_ksc<16>(ChainGeom<16>::MINB) : (max_rank <= 32 ? chain_ksc<32>(ChainGeom<32>::MINB) : chain_ksc<64>(ChainGeom<64>::MINB));
-    return c < ksc ? c : ksc;
-}
 
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s)
 {

@@ -276,25 +276,11 @@ int mlora_assist_import(int n_proj, void *const *res, const void *const *out_slo
     return MLORA_OK;
 }
 
-int mlora_set_option(int option, int value)
-{
-    mlora::DecodeOptions &o = mlora::decode_options();
-    switch (option) {
-    case MLORA_OPT_DECODE_ONE_LAUNCH: o.chain = value ? 1 : 0; return MLORA_OK;
-    case MLORA_OPT_DECODE_SPIN_LIMIT: o.spin_limit = value; return MLORA_OK;
-    case MLORA_OPT_DECODE_GRID_CAP:
-        if (value < 64 || value > (1 << 20)) return fail(MLORA_ERANGE, "grid cap must be in 64..1048576 (got %d)", value);
-        o.grid_cap = value;
-        return MLORA_OK;
-    default: return fail(MLORA_EINVAL, "unknown option %d", option);
-    }
-}
-
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank)
 {
     if (n_proj < 1 || T < 1 || max_hin < 1) return 0;
-    // slots of the narrowest shrink slice any launch form uses at this rank
-    const int ksc = mlora::bgmv_min_slice_chunks(max_rank);
+    int ksc, nte;
+    mlora::bgmv_split_slices(max_rank, &ksc, &nte);
     const int64_t ks = (max_hin + ksc * 8 - 1) / (ksc * 8);
     return (int64_t)n_proj * T * ks * mlora::bgmv_split_rank_stride(max_rank) * (int64_t)sizeof(float);
 }
@@ -373,7 +359,6 @@ static int bgmv_multi_impl(int n_proj, void *const *y, const void *const *x, con
             ex += (hout[p] + nte * 8 - 1) / (nte * 8);
             a.sh_end[p] = sh; a.ex_end[p] = ex;
         }
-        a.chain_ok = 1;                       // the workspace holds the one-launch form's slots as well
         rc = mlora::launch_bgmv_split(a, dtype, group, max_rank, static_cast<hipStream_t>(stream));
     } else {
         rc = mlora::launch_bgmv(a, dtype, group, max_rank, false, static_cast<hipStream_t>(stream));

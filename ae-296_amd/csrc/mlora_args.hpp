@@ -10,13 +10,8 @@ constexpr int MAX_PROJ = 8;
 constexpr int MAX_RANK = 64;
 // Decode work record (int32 words): [0] tokens in the item (0 = empty), [1] adapter (-1 = none),
 // [2] rank, [3] scaling (float bits), [4..11] token ids, [12..15] zero, [16..79] row of rank row j (-1 = absent).
-// The last record of a plan (index work_cap - 1, never a work item: 0 tokens) is a trailer: [16] work items in the
-// list, [17..20] how many of them fall into each rank bucket, [21] 1 when the list is ordered by bucket.
 constexpr int WORK_WORDS = 80;
 constexpr int WORK_ROWS_AT = 16;
-constexpr int WORK_BUCKETS = 4;
-// Rank bucket of a work item: 0 = more than 32 rank rows, 1 = 17..32, 2 = 9..16, 3 = at most 8.
-__host__ __device__ inline int work_bucket(int rank) { return rank > 32 ? 0 : (rank > 16 ? 1 : (rank > 8 ? 2 : 3)); }
 // Prefill tile record (int32 words): [0] tokens in the tile (0 = nothing to do), [1] adapter (-1 = none),
 // [2] rank, [3] scaling (float bits), [4] first token, [5] segment, [6..15] zero, [16..79] row of rank row j.
 constexpr int TILE_WORDS = 80;
@@ -37,15 +32,6 @@ struct PoolView {
     long long n_rows_b;
     long long a_dense_stride;  // rows between adapters when a_tbl == nullptr
     long long b_dense_stride;  // rows (B as rank rows) or elements (B^T blocks) when b_tbl == nullptr
-};
-
-// One-launch ("chained") decode form: the shrink units come first in the grid, the expand units after them; an expand
-// unit waits for the arrival counter of its (record, projection) in the record's words 12..15.
-struct ChainArgs {
-    int grid_sh, grid_ex;                      // workgroups of the shrink part / of the expand part
-    int spin_limit;                            // polls of an expand workgroup before it computes the sums itself (< 0: none)
-    int sh_end[WORK_BUCKETS][MAX_PROJ];        // shrink units of projections 0..p, for an item of rank bucket k
-    int ex_end[WORK_BUCKETS][MAX_PROJ];        // expand units likewise
 };
 
 struct BgmvArgs {
@@ -76,8 +62,6 @@ struct BgmvArgs {
     // two-launch form: records the shrink / expand grid covers; a workgroup walks records b, b + stride, ... < items_cap
     // (set by the launcher)
     int rec_stride_sh, rec_stride_ex;
-    int chain_ok;                  // the caller allows the one-launch form (its workspace is sized for it)
-    ChainArgs chain;               // one-launch form (set by the launcher)
 };
 
 constexpr int SCATTER_MAX_JOBS = 16;
@@ -204,11 +188,6 @@ struct GemmLoraArgs {
 int launch_bgmv(const BgmvArgs &a, int dtype, int group, int max_rank, bool b_transposed, hipStream_t s);
 int launch_bgmv_split(const BgmvArgs &a, int dtype, int group, int max_rank, hipStream_t s);   // a.b_transposed: max_rank is the pool's rank (8, 16, 32 or 64)
 int bgmv_split_rank_stride(int max_rank);
-int bgmv_min_slice_chunks(int max_rank);
-// Decode launch options (process-wide, set through mlora_set_option): whether calls of about one round of
-// workgroups run as the one-launch chained form, its spin limit and the cap on the workgroups of each part.
-struct DecodeOptions { int chain; int spin_limit; int grid_cap; };
-DecodeOptions &decode_options();
 void bgmv_split_slices(int max_rank, int *shrink_chunks, int *expand_chunks, bool transposed_b = false);   // slice widths in 16-byte chunks
 int launch_gather(const GatherArgs &a, hipStream_t s);
 int launch_scatter(const ScatterArgs &a, hipStream_t s);

@@ -238,53 +238,37 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
         }
     }
     // ---- decode work records, in launch order: the records in use first; records b, b + 8, ... hold consecutive
-    // positions of the list (the one-launch fused decode form, whose workgroup b of a projection reads record b,
-    // runs them on one XCD: workgroups are dealt to the 8 XCDs round-robin; the other forms take the records in
-    // order).  Batches beyond 2048 tokens (chunk headers not in LDS) keep plain chunk order.
+    // chunks (the one-launch decode form, whose workgroup b of a projection reads record b, runs them on one XCD:
+    // workgroups are dealt to the 8 XCDs round-robin; the two-launch form takes the records in order).  Batches
+    // beyond 2048 tokens (chunk headers not in LDS) keep plain chunk order inside each range.
     if (g.work) {
         __shared__ int s_nchunks;
-        __shared__ int s_nb[WORK_BUCKETS];       // chunks per rank bucket
         if (tid == GATHER_NT - 1) s_nchunks = ch_incl;
-        if (tid < WORK_BUCKETS) s_nb[tid] = 0;
         __syncthreads();                         // chunk_* arrays written above are visible to the whole block
         const int n_chunks = s_nchunks;
         const int per_xcd = (n_chunks + 7) >> 3;
         if constexpr (LDS_HDR) {
-            // The list is ordered by rank bucket (more than 32 rank rows, 17..32, 9..16, at most 8; chunks without
-            // adapter count as rank 0), ties in chunk order, so that the chunks of one adapter stay next to each
-            // other: the workgroups of the wide items are dispatched first, and a kernel that is told the number
-            // of chunks per bucket (trailer record) can number its units of work without reading a record.  A
-            // stable partition: every thread owns EPT consecutive chunks, two block scans over packed counts.
+            // Within each of the eight ranges of chunks the records are written in order of falling rank
+            // (ties keep chunk order, so the chunks of one adapter stay next to each other): the workgroups of
+            // the wide items are then dispatched first and the narrow ones fill in behind them.  A counting sort:
+            // chunks per (XCD, rank), then one thread per (XCD, rank) places its chunks.
             __shared__ int s_ord[MAXT];
-            int differs = 0;                     // a list of one bucket keeps chunk order and skips the partition
-            for (int c = tid; c < n_chunks; c += GATHER_NT)
-                differs |= work_bucket(s_chdr[c] >> (TOK_BITS + 4)) != work_bucket(s_chdr[0] >> (TOK_BITS + 4));
+            __shared__ int s_cntx[8][MAX_RANK + 1];
+            int differs = 0;                     // a pool of one rank keeps chunk order and skips the sort
+            for (int c = tid; c < n_chunks; c += GATHER_NT) differs |= (s_chdr[c] >> (TOK_BITS + 4)) != (s_chdr[0] >> (TOK_BITS + 4));
+            for (int i = tid; i < 8 * (MAX_RANK + 1); i += GATHER_NT) (&s_cntx[0][0])[i] = 0;
             const bool mixed = __syncthreads_or(differs) != 0;
-            int bk[EPT], lo01 = 0, lo23 = 0;
-#pragma unroll
-            for (int e = 0; e < EPT; e++) {
-                const int c = base + e;
-                bk[e] = c < n_chunks ? work_bucket(s_chdr[c] >> (TOK_BITS + 4)) : -1;
-                lo01 += (bk[e] == 0 ? 1 : 0) + (bk[e] == 1 ? 1 << 16 : 0);
-                lo23 += (bk[e] == 2 ? 1 : 0) + (bk[e] == 3 ? 1 << 16 : 0);
-            }
-            const int in01 = block_scan_inclusive<0>(lo01, 0, s_wave);
-            const int in23 = block_scan_inclusive<0>(lo23, 0, s_wave);
-            if (tid == GATHER_NT - 1) {
-                s_nb[0] = in01 & 0xffff; s_nb[1] = in01 >> 16; s_nb[2] = in23 & 0xffff; s_nb[3] = in23 >> 16;
-            }
+            if (mixed)
+                for (int c = tid; c < n_chunks; c += GATHER_NT) atomicAdd(&s_cntx[c / per_xcd][s_chdr[c] >> (TOK_BITS + 4)], 1);
             __syncthreads();
-            if (mixed) {
-                int at0 = (in01 - lo01) & 0xffff;
-                int at1 = s_nb[0] + ((in01 - lo01) >> 16);
-                int at2 = s_nb[0] + s_nb[1] + ((in23 - lo23) & 0xffff);
-                int at3 = s_nb[0] + s_nb[1] + s_nb[2] + ((in23 - lo23) >> 16);
-#pragma unroll
-                for (int e = 0; e < EPT; e++) {
-                    if (bk[e] == 0) s_ord[at0++] = base + e;
-                    else if (bk[e] == 1) s_ord[at1++] = base + e;
-                    else if (bk[e] == 2) s_ord[at2++] = base + e;
-                    else if (bk[e] == 3) s_ord[at3++] = base + e;
+            if (mixed && tid < 8 * (MAX_RANK + 1)) {
+                const int xcd = tid / (MAX_RANK + 1), rk = tid - xcd * (MAX_RANK + 1);
+                if (s_cntx[xcd][rk] > 0) {
+                    int at = xcd * per_xcd;
+                    for (int r2 = rk + 1; r2 <= MAX_RANK; r2++) at += s_cntx[xcd][r2];
+                    const int lo = xcd * per_xcd, hi = lo + per_xcd < n_chunks ? lo + per_xcd : n_chunks;
+                    for (int c = lo; c < hi; c++)
+                        if ((s_chdr[c] >> (TOK_BITS + 4)) == rk) s_ord[at++] = c;
                 }
             }
             __syncthreads();
@@ -298,11 +282,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
                 const int b = q / QPR, w4 = q - b * QPR;
                 const int pos = (b & 7) * per_xcd + (b >> 3);
                 int4 v = make_int4(0, w4 == 0 ? -1 : 0, 0, 0);
-                if (b == g.work_cap - 1) {
-                    // trailer: never a work item (no tokens); words 16.. hold the list's length and its buckets
-                    if (w4 == WORK_ROWS_AT / 4) v = make_int4(n_chunks, s_nb[0], s_nb[1], s_nb[2]);
-                    else if (w4 == WORK_ROWS_AT / 4 + 1) v = make_int4(s_nb[3], 1, 0, 0);
-                } else if ((b >> 3) < per_xcd && pos < n_chunks) {
+                if ((b >> 3) < per_xcd && pos < n_chunks) {
                     const int c = mixed ? s_ord[pos] : pos;
                     const int hdr = s_chdr[c];
                     const int start = hdr & (int)tmask, len = (hdr >> TOK_BITS) & 15, rk = hdr >> (TOK_BITS + 4);
@@ -334,10 +314,7 @@ __global__ __launch_bounds__(GATHER_NT) void gather_kernel(const GatherArgs g)
             const int b = (int)(idx / WORK_WORDS), w = (int)(idx - (long long)b * WORK_WORDS);
             const int c = (b & 7) * per_xcd + (b >> 3);
             int val = w == 1 ? -1 : 0;
-            if (b == g.work_cap - 1) {
-                // trailer: the list's length; no bucket counts (word 21 = 0: the list is in plain chunk order)
-                if (w == WORK_ROWS_AT) val = n_chunks;
-            } else if ((b >> 3) < per_xcd && c < n_chunks) {
+            if ((b >> 3) < per_xcd && c < n_chunks) {
                 const int start = g.chunk_start[c], len = g.chunk_len[c], a = g.chunk_adapter[c];
                 int rk = 0;
                 if (a >= 0) { rk = gather_rank(g, a); rk = rk < 0 ? 0 : (rk > MAX_RANK ? MAX_RANK : rk); }

@@ -25,12 +25,10 @@ CNT_NSEG, CNT_NVALID, CNT_NCHUNK, CNT_BAD, CNT_WORDS = 0, 1, 2, 3, 8
 WORK_WORDS = 80
 SCATTER_MAX_JOBS = 16
 NOALLOC_SCRATCH_BYTES = 16 << 20    # MLORA_NOALLOC_SCRATCH_BYTES
-OPT_DECODE_ONE_LAUNCH, OPT_DECODE_SPIN_LIMIT, OPT_DECODE_GRID_CAP = 1, 2, 3
 
 
 def work_cap(T: int) -> int:
-    """MLORA_WORK_CAP(T): records of a decode plan, the last one being the trailer."""
-    return ((T + 7) // 8) * 8 + 8
+    return ((T + 7) // 8) * 8
 
 
 _vp, _i32, _i64, _f32 = C.c_void_p, C.c_int, C.c_int64, C.c_float
@@ -46,7 +44,6 @@ SIGNATURES = {
     "mlora_host_free": (_i32, [_vp]),
     "mlora_assist_export": (_i32, [_vp, _i32, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),
     "mlora_assist_import": (_i32, [_i32, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
-    "mlora_set_option": (_i32, [_i32, _i32]),
     "mlora_bgmv_workspace_bytes": (_i64, [_i32, _i32, _i32, _i32]),
     "mlora_bgmv_multi": (_i32, [_i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp, _i32, _i32, _i32,
                                 _i64, _i32, _vp, _i32, _vp, _i64, _i32, _i32, _vp]),

@@ -70,7 +70,7 @@ extern "C" {
 /* Decode work records written by mlora_pool_gather and read by mlora_bgmv_multi: one record of
  * MLORA_WORK_WORDS int32 per workgroup and projection, MLORA_WORK_CAP(T) records per batch. */
 #define MLORA_WORK_WORDS 80
-#define MLORA_WORK_CAP(T) ((((T) + 7) / 8) * 8 + 8)   /* the last record is a trailer, see mlora_pool_gather */
+#define MLORA_WORK_CAP(T) ((((T) + 7) / 8) * 8)
 
 const char *mlora_last_error(void);
 int mlora_version(void);
@@ -94,17 +94,12 @@ int mlora_version(void);
  *                       (c mod P) * 8 + c / P with P = ceil(n_chunks / 8): the records in use come first,
  *                       records b, b + 8, ... hold a range of P consecutive chunks (the one-launch decode
  *                       form runs such a range on one XCD; the two-launch form takes the records in
- *                       order).  For T <= 2048 the list is the chunk list ordered by rank bucket (more than
- *                       32 rank rows, 17..32, 9..16, at most 8; chunks without adapter count as rank 0), ties
- *                       in chunk order, which starts the workgroups of wide items first; the chunk_* arrays
- *                       keep chunk order.  Record words:
+ *                       order).  For T <= 2048 the chunks of each such range are placed by falling rank
+ *                       (ties in chunk order), which starts the workgroups of wide items first; the
+ *                       chunk_* arrays keep chunk order.  Record words:
  *                       [0] tokens (0 = empty record) [1] adapter [2] rank [3] scaling (float bits)
  *                       [4..11] token ids [12..15] 0 [16..79] row of rank row j in a rows slab, -1 if
- *                       j >= rank or the page id is outside [0, n_pages).  Words 12..15 are arrival
- *                       counters of the one-launch decode form of mlora_bgmv_multi, which leaves them 0.
- *                       The last record (index MLORA_WORK_CAP(T) - 1) is a trailer, never a work item
- *                       (0 tokens): [16] records in use, [17..20] how many of them fall into each rank
- *                       bucket, [21] 1 when the list is ordered by bucket (T <= 2048), else 0.
+ *                       j >= rank or the page id is outside [0, n_pages).
  * T <= MLORA_GATHER_MAX_T.  All outputs are exact integers / copied floats (bit-exact).
  */
 int mlora_pool_gather(const int32_t *tok_adapter, int T,
@@ -182,19 +177,7 @@ int mlora_assist_import(int n_proj, void *const *res, const void *const *out_slo
  * records than MLORA_WORK_CAP(T): a workgroup serves records b, b + stride, ... of its residue mod 8 and stops
  * at the first empty one.  The layout mlora_pool_gather writes (records in use of each residue first) is what
  * makes that valid; a caller that fills `work` itself must keep it.
- * One-launch form: a call with workspace whose batch makes for about one round of workgroups (T <= 2048, group <= 4)
- * runs as ONE launch in which the expand workgroups follow the shrink workgroups in the grid, request their B and
- * y rows at once and wait (bounded) for the arrival counter of their item in words 12..15 of its work record; the
- * counters are left at zero.  The records are therefore written to by the call although they are inputs: calls
- * that use the same records must be ordered on one stream (as calls that share a workspace already must).
- * mlora_set_option(MLORA_OPT_DECODE_ONE_LAUNCH, 0) keeps such calls on the two launches.
  */
-#define MLORA_OPT_DECODE_ONE_LAUNCH 1   /* 1 (default): calls of about one round of workgroups run as one launch */
-#define MLORA_OPT_DECODE_SPIN_LIMIT 2   /* polls of a waiting expand workgroup before it computes the sums itself (default 2^20; <= 0: none) */
-#define MLORA_OPT_DECODE_GRID_CAP 3     /* most workgroups each part of the one-launch form may have (default 2048) */
-/* Process-wide launch options of the decode call (no counterpart in the reference). */
-int mlora_set_option(int option, int value);
-
 int64_t mlora_bgmv_workspace_bytes(int n_proj, int T, int max_hin, int max_rank);
 int mlora_bgmv_multi(int n_proj, void *const *y, const void *const *x,
                      const void *const *a_rows, const void *const *b_rows,

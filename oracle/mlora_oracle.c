@@ -234,12 +234,9 @@ int orc_build_chunks(const int32_t *seg_start, const int32_t *seg_len, const int
     return ORC_OK;
 }
 
-/* Decode work records, in launch order.  Position c of the list is served by the
+/* Decode work records for the fused decode kernel, in launch order.  Chunk c is served by the
  * workgroup b = (c mod per_xcd) * 8 + c / per_xcd with per_xcd = ceil(n_chunks / 8): workgroups are
- * dealt to the 8 XCDs round-robin by id, so consecutive positions land on one XCD.  The list is the chunk
- * list, for batches of at most 2048 tokens ordered by rank bucket (more than 32 rank rows, 17..32, 9..16,
- * at most 8; chunks without adapter count as rank 0), ties in chunk order.  The last record (work_cap - 1)
- * is a trailer with 0 tokens: [16] chunks, [17..20] chunks per bucket, [21] 1 when ordered by bucket.  Record b
+ * dealt to the 8 XCDs round-robin by id, so consecutive chunks land on one XCD.  Record b
  * (ORC_WORK_WORDS int32): [0] tokens in the chunk (0 = empty record), [1] adapter (-1 = none),
  * [2] rank clamped to 0..64, [3] scaling as float bits, [4..11] token ids (-1 unused), [12..15] 0,
  * [16..79] row of rank row j = page_tbl[a][j / page_rows] * page_rows + j % page_rows, or -1 when
@@ -251,13 +248,15 @@ int orc_build_work(const int32_t *chunk_start, const int32_t *chunk_len, const i
                    const float *scaling, int max_pages, int page_rows, int64_t n_pages,
                    int work_cap, int32_t *work /* [work_cap * ORC_WORK_WORDS] */)
 {
-    if (work_cap < 8 || (work_cap & 7) || n_chunks > work_cap - 8) return ORC_EINVAL;
+    if (work_cap < 0 || (work_cap & 7) || n_chunks > work_cap) return ORC_EINVAL;
     int per_xcd = (n_chunks + 7) / 8;
     for (int b = 0; b < work_cap; b++) {
         int32_t *w = work + (size_t)b * ORC_WORK_WORDS;
         for (int i = 0; i < ORC_WORK_WORDS; i++) w[i] = 0;
         w[1] = -1;
     }
+    /* Batches of at most 2048 tokens (work_cap <= 2048): inside the range of chunks that goes to one XCD the
+     * records follow falling rank, ties in chunk order (a stable insertion sort per range). */
     int *ord = (int *)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(int));
     int *crk = (int *)malloc((size_t)(n_chunks > 0 ? n_chunks : 1) * sizeof(int));
     if (!ord || !crk) { free(ord); free(crk); return ORC_EINVAL; }
@@ -267,22 +266,15 @@ int orc_build_work(const int32_t *chunk_start, const int32_t *chunk_len, const i
         crk[c] = rk;
         ord[c] = c;
     }
-    int nb[4] = {0, 0, 0, 0};
-    const int ordered = work_cap <= 2048 + 8;
-    if (ordered) {
-        /* stable partition by bucket */
-        int at = 0;
-        for (int k = 0; k < 4; k++)
-            for (int c = 0; c < n_chunks; c++) {
-                int rk = crk[c];
-                int bk = rk > 32 ? 0 : (rk > 16 ? 1 : (rk > 8 ? 2 : 3));
-                if (bk == k) { ord[at++] = c; nb[k]++; }
+    if (work_cap <= 2048) {
+        for (int lo = 0; lo < n_chunks; lo += per_xcd) {
+            int hi = lo + per_xcd < n_chunks ? lo + per_xcd : n_chunks;
+            for (int i = lo + 1; i < hi; i++) {
+                int c = ord[i], j = i;
+                while (j > lo && crk[ord[j - 1]] < crk[c]) { ord[j] = ord[j - 1]; j--; }
+                ord[j] = c;
             }
-    }
-    {
-        int32_t *tr = work + (size_t)(work_cap - 1) * ORC_WORK_WORDS;
-        tr[16] = n_chunks;
-        if (ordered) { tr[17] = nb[0]; tr[18] = nb[1]; tr[19] = nb[2]; tr[20] = nb[3]; tr[21] = 1; }
+        }
     }
     for (int pos = 0; pos < n_chunks; pos++) {
         int c = ord[pos];

@@ -140,8 +140,7 @@ WORK_WORDS = 80
 
 
 def work_cap(T):
-    """Records of a decode plan for T tokens: T rounded up to 8, plus 8 whose last one is the trailer."""
-    return ((T + 7) // 8) * 8 + 8
+    return ((T + 7) // 8) * 8
 
 
 def build_work(chunk_start, chunk_len, chunk_adapter, perm, page_tbl, rank, scaling, page_rows, n_pages, T):

@@ -92,17 +92,16 @@ def test_build_chunks_brute_force(toks, group):
     assert len(cs) <= max(T, 1)
 
 
-def _bucket(r):
-    return 0 if r > 32 else 1 if r > 16 else 2 if r > 8 else 3
-
-
-def _record_order(ca, rank, heavy_first):
+def _record_order(ca, rank, P, heavy_first):
     """Chunk held by every position of the record sequence: chunk order, and for batches of at most 2048 tokens
-    ordered by rank bucket (> 32, 17..32, 9..16, <= 8 rank rows; no adapter = rank 0), ties in chunk order
-    (numpy's stable argsort)."""
+    falling rank inside each range of P chunks (one XCD), ties in chunk order (numpy's stable argsort)."""
+    n = len(ca)
     crk = np.array([min(max(int(rank[a]), 0), 64) if a >= 0 else 0 for a in ca], dtype=np.int64)
-    bk = np.array([_bucket(r) for r in crk], dtype=np.int64)
-    return list(np.argsort(bk, kind="stable")) if heavy_first else list(range(len(ca))), bk
+    order = []
+    for lo in range(0, n, max(P, 1)):
+        idx = np.arange(lo, min(lo + P, n))
+        order += list(idx[np.argsort(-crk[idx], kind="stable")] if heavy_first else idx)
+    return order
 
 
 def test_build_work_by_enumeration():
@@ -118,21 +117,18 @@ def test_build_work_by_enumeration():
     perm, ss, sl, sa, nv = orc.build_segments(tok, N)
     cs, cl, ca = orc.build_chunks(ss, sl, sa, nv, T, group)
     work = orc.build_work(cs, cl, ca, perm, page_tbl, rank, scaling, page_rows, n_pages, T)
-    cap = ((T + 7) // 8) * 8 + 8
+    cap = ((T + 7) // 8) * 8
     assert work.shape == (cap, orc.WORK_WORDS)
     P = -(-len(cs) // 8)
     used = set()
-    order, bk = _record_order(ca, rank, heavy_first=True)
+    order = _record_order(ca, rank, P, heavy_first=True)
     assert sorted(order) == list(range(len(cs)))
-    # wide buckets first, chunk order inside a bucket
+    # heavy first inside a range, and a range keeps its chunks (one XCD, residue pos // P)
     for pos in range(1, len(order)):
-        assert (bk[order[pos - 1]], order[pos - 1]) < (bk[order[pos]], order[pos])
-    assert len(set(bk)) > 2                       # the case has several buckets and chunks without adapter
-    # the trailer: list length, chunks per bucket, "ordered" flag; no tokens, so no kernel treats it as an item
-    tr = work[cap - 1]
-    assert tr[0] == 0 and tr[1] == -1 and np.all(tr[2:16] == 0)
-    assert tr[16] == len(cs) and tr[17:21].tolist() == [int((bk == k).sum()) for k in range(4)] and tr[21] == 1
-    assert np.all(tr[22:] == 0)
+        if pos % P:
+            ra, rb = (rank[ca[order[k]]] if ca[order[k]] >= 0 else 0 for k in (pos - 1, pos))
+            assert ra >= rb
+    assert all(order[pos] // P == pos // P for pos in range(len(order)))
     for pos, c in enumerate(order):
         b = (pos % P) * 8 + pos // P
         used.add(b)
@@ -151,7 +147,7 @@ def test_build_work_by_enumeration():
             assert w[16 + j] == want
     # consecutive positions of a range share blockIdx mod 8 (one XCD): position pos sits at residue pos // P
     assert all(((pos % P) * 8 + pos // P) % 8 == pos // P for pos in range(len(cs)))
-    for b in range(cap - 1):
+    for b in range(cap):
         if b not in used:
             assert work[b, 0] == 0 and work[b, 1] == -1 and np.all(work[b, 2:] == 0)
 
@@ -170,8 +166,6 @@ def test_build_work_keeps_chunk_order_beyond_2048_tokens():
     for c in range(len(cs)):
         w = work[(c % P) * 8 + c // P]
         assert w[0] == cl[c] and w[1] == ca[c] and w[4] == perm[cs[c]]
-    tr = work[-1]
-    assert tr[0] == 0 and tr[16] == len(cs) and np.all(tr[17:] == 0)      # no bucket counts: plain chunk order
 
 
 def test_sgmv_plan_brute_force():
