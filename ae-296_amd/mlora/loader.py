@@ -133,21 +133,25 @@ class AdapterLoader:
         return HostAdapter(rank, float(scaling), blob, offsets)
 
     # ------------------------------------------------------------------ device side
-    def load_async(self, slot: int, host: HostAdapter, pages: Optional[Sequence[int]] = None) -> LoadTicket:
+    def load_async(self, slot: int, host: HostAdapter, pages: Optional[Sequence[int]] = None,
+                   first_layer: Optional[int] = None, layers_per_copy: Optional[int] = None) -> LoadTicket:
         """Bind `slot` to the adapter (page-table update) and start moving its rows into the pool.
-        Returns at once; nothing on the caller's streams waits unless it asks the ticket to."""
+        Returns at once; nothing on the caller's streams waits unless it asks the ticket to.  `first_layer` and
+        `layers_per_copy` override the loader's own for this load (layer 0 first, in small groups, suits a consumer
+        that walks the layers in order and waits for each: `ticket.wait_layer`)."""
         pool = self.pool
+        per_copy = self.layers_per_copy if layers_per_copy is None else max(1, int(layers_per_copy))
         page_ids = pool.allocate(slot, host.rank, host.scaling, pages)
         pages_c = (C.c_int32 * len(page_ids))(*[int(v) for v in page_ids])
-        order = layer_order(pool.n_layers, self.first_layer)
+        order = layer_order(pool.n_layers, self.first_layer if first_layer is None else first_layer)
         ticket = LoadTicket(slot, order, {})
         layer_elems = host.blob.shape[1]
         lib = _ext.lib()
         esz = host.blob.element_size()
         self.stream.wait_stream(torch.cuda.current_stream())          # rows of an evicted adapter may still be in use
         with torch.cuda.stream(self.stream):
-            for g0 in range(0, len(order), self.layers_per_copy):
-                group = order[g0:g0 + self.layers_per_copy]
+            for g0 in range(0, len(order), per_copy):
+                group = order[g0:g0 + per_copy]
                 # consecutive layers travel as one copy
                 runs, start = [], 0
                 for i in range(1, len(group) + 1):

@@ -144,18 +144,35 @@ class Lora_CPU:
     def results_ready(self) -> bool:
         return not self.np_signal[:, :self.active_cpu].any()
 
-    def collect_qkv(self, tkn_num: int, batch_size: int, timeout_s: Optional[float] = 60.0) -> List[torch.Tensor]:
-        """Wait until every active worker has reset its signal, then bring the rank's column slice of the
-        q, k and v results to the device as ``[batch_size, tkn_num, out_size]`` tensors (one launch)."""
+    def collect_each(self, tkn_num: int, batch_size: int, timeout_s: Optional[float] = 60.0):
+        """Yields ``(projection index, result [batch_size, tkn_num, out_size])`` for q, k and v, each as soon as all of
+        its workers have reset their signals: that projection's rows come to the device (one launch) while the
+        workers of the others are still computing -- the reference brings chunks back as they finish
+        (``lora_cpu.py:219-270``)."""
         t0 = time.perf_counter()
-        while not self.results_ready():
-            if timeout_s is not None and time.perf_counter() - t0 > timeout_s:
+        lib = _ext.lib()
+        pending = [0, 1, 2]
+        while pending:
+            progressed = False
+            for q in list(pending):
+                if self.np_signal[q, :self.active_cpu].any():
+                    continue
+                res = torch.empty((batch_size, tkn_num, self.out_size), dtype=self._dtype, device=self.device)
+                rp = (C.c_void_p * 4)(res.data_ptr(), None, None, None)
+                op = (C.c_void_p * 4)(self._out[q].dev_ptr, None, None, None)
+                _ext.check(lib.mlora_assist_import(1, rp, op, batch_size, tkn_num, self.hidden_dim, self.out_size,
+                                                   self.out_size * self.gpu_id, self.lora_num, PROMPT_MAX_LENGTH,
+                                                   _ext.current_stream_ptr()))
+                pending.remove(q)
+                progressed = True
+                yield q, res
+            if pending and not progressed and timeout_s is not None and time.perf_counter() - t0 > timeout_s:
                 raise TimeoutError("CPU workers did not finish in time")
-        res = [torch.empty((batch_size, tkn_num, self.out_size), dtype=self._dtype, device=self.device) for _ in range(3)]
-        rp = (C.c_void_p * 4)(*[r.data_ptr() for r in res], None)
-        op = (C.c_void_p * 4)(*[o.dev_ptr for o in self._out], None)
-        rc = _ext.lib().mlora_assist_import(3, rp, op, batch_size, tkn_num, self.hidden_dim, self.out_size,
-                                            self.out_size * self.gpu_id, self.lora_num, PROMPT_MAX_LENGTH,
-                                            _ext.current_stream_ptr())
-        _ext.check(rc)
+
+    def collect_qkv(self, tkn_num: int, batch_size: int, timeout_s: Optional[float] = 60.0) -> List[torch.Tensor]:
+        """The q, k and v results of the batch in flight as ``[batch_size, tkn_num, out_size]`` tensors (the rank's
+        column slice), each imported as soon as its projection's workers are done."""
+        res: List[Optional[torch.Tensor]] = [None, None, None]
+        for q, r in self.collect_each(tkn_num, batch_size, timeout_s):
+            res[q] = r
         return res
