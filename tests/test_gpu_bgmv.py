@@ -358,6 +358,7 @@ MANY_ROUNDS = [
     (2, [8, 16, 32], 8192, 2048, 1200, FP16),
     (1, [16, 64], 8192, 2048, 600, BF16),
     (8, [8, 16], 16384, 4096, 1200, BF16),
+    (8, [8, 16, 32], 8192, 2048, 1200, FP16),
 ]
 
 
