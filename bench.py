@@ -1120,6 +1120,9 @@ def main():
         flat[f"{w}_ms_per_step"] = leg["ms_per_step"]
         if rf["bound"] == "hbm":
             flat[f"{w}_hbm_frac"] = rf["frac"]
+        if w == "c1":
+            # 2.9 MB per call = 0.36 us at the HBM peak: a single launch cannot be that short, whatever the kernel
+            flat["c1_note"] = "latency-scale op: bounded by one kernel launch, not by HBM"
         if "launch_us" in rf:
             flat[f"{w}_launch_us"] = rf["launch_us"]
         if w == "c4":
@@ -1133,9 +1136,10 @@ def main():
             for k in ("cached_ms", "cpu_assisted_ms", "on_demand_ms", "pipelined_ms", "ordering_holds"):
                 flat[f"coldstart_{k}"] = leg.get(k)
     flat["bench_wall_s"] = time.perf_counter() - t_start
-    # key order of the printed line: the legs first, the headline's own fields (and the flat scalars) last
+    # key order of the printed line: the legs first, the headline's own fields after them, `config` (with the flat scalars) last
     ordered = {"legs": legs}
-    ordered.update(line)
+    ordered.update({k: v for k, v in line.items() if k != "config"})
+    ordered["config"] = line["config"]
     print(json.dumps(ordered), flush=True)
 
 
