@@ -61,7 +61,8 @@ class ColdStartPrefill:
         self.slot_adapter = np.zeros(cpu.lora_num, np.int32)
         self.host: Dict[int, HostAdapter] = {}
         self.resident: Dict[int, int] = {}            # adapter id -> pool slot
-        self.tickets: List[LoadTicket] = []
+        self.tickets: List[LoadTicket] = []           # loads the batch in flight depends on
+        self._loading: Dict[int, LoadTicket] = {}     # adapter id -> its load, until it is seen complete
         self.count_use_gpu_lora = 0                   # transformer_layer_infer.py:117-118
         self.count_use_cpu_lora = 0
         self._batch = None
@@ -92,7 +93,10 @@ class ColdStartPrefill:
         return self.cpu.stop_workers()
 
     def evict(self, aid: int) -> None:
+        """Give the adapter's pages back.  A load of it that is still running finishes on the loader's stream first
+        (the next load into these pages is queued behind it); no batch that uses the adapter may be in flight."""
         slot = self.resident.pop(aid, None)
+        self._loading.pop(aid, None)
         if slot is not None:
             self.pool.release(slot)
 
@@ -108,20 +112,37 @@ class ColdStartPrefill:
         self.tickets = []
         slots = []
         for b, aid in enumerate(adapter_ids):
+            if aid not in self.host:
+                raise KeyError(f"adapter {aid} was never registered")
             if aid in self.resident:
                 slots.append(self.resident[aid])
+                t = self._loading.get(aid)
+                if t is not None:
+                    # bound to a slot by an earlier batch and possibly still on its way: this batch depends on that load too
+                    if t.progress() == 0:
+                        del self._loading[aid]
+                    elif t not in self.tickets:
+                        self.tickets.append(t)
                 continue
             if mode == "cached":
                 raise RuntimeError(f"adapter {aid} is not resident")
             used = set(self.resident.values())
-            slot = next(s for s in range(self.pool.n_slots) if s not in used)
+            slot = next((s for s in range(self.pool.n_slots) if s not in used), None)
+            if slot is None:
+                raise RuntimeError(f"no free slot for adapter {aid}: evict one of {sorted(self.resident)} first")
             order = dict(first_layer=0, layers_per_copy=2) if mode == "pipelined" else {}
-            self.tickets.append(self.loader.load_async(slot, self.host[aid], **order))    # the router's progress = 1 (manager.py:178-181)
+            t = self.loader.load_async(slot, self.host[aid], **order)    # the router's progress = 1 (manager.py:178-181)
+            self.tickets.append(t)
+            self._loading[aid] = t
             self.resident[aid] = slot
             slots.append(slot)
-        if mode == "on_demand":
+        if mode in ("on_demand", "cached"):
+            # on demand: the prefill starts when the adapters are in.  cached: they are, unless an earlier batch started
+            # a load that has not finished -- then this one waits for it the same way
             for t in self.tickets:
                 t.wait()
+            for aid in adapter_ids:
+                self._loading.pop(aid, None)
             self.tickets = []
         dev = self.pool.device
         seg_start = torch.arange(0, B * tkn, tkn, dtype=torch.int32, device=dev)
@@ -144,7 +165,7 @@ class ColdStartPrefill:
         path = force or ("gpu" if (self._mode == "pipelined" or self.use_gpu_pipeline(layer)) else "cpu")
         if path == "gpu":
             for t in self.tickets:
-                t.wait_layer(layer)               # orders the stream after the rows' arrival (already past, unless pipelined)
+                t.wait_layer(layer)               # orders the stream after the rows' arrival (already past, unless pipelined or forced)
             self.count_use_gpu_lora += 1
         else:
             L = self.pool.n_layers

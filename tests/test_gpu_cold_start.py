@@ -190,3 +190,54 @@ def test_cold_start_free_running():
     finally:
         cs.stop_workers()
         cpu.close()
+
+
+def test_cold_start_next_batch_while_the_load_is_in_flight():
+    """A second batch on an adapter whose load an earlier batch started depends on that load too: it may not read the
+    pool before the rows are in (forced GPU path: the launch waits on the device; cached: the host waits).  A batch
+    that needs a slot when none is free says so."""
+    pool, cpu, cs, weights = _setup(5)
+    scalings = {a: (2.0 if a % 2 == 0 else 0.5) for a in range(5)}
+    tkn = 8
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(tkn, H, device="cuda", generator=gen).half()
+    y0 = [torch.randn(tkn, H, device="cuda", generator=gen).half() for _ in NAMES]
+    gate_host = torch.empty(1 << 29, dtype=torch.uint8, pin_memory=True)
+    gate_dev = torch.empty(1 << 29, dtype=torch.uint8, device="cuda")
+    try:
+        torch.cuda.synchronize()
+        with torch.cuda.stream(cs.loader.stream):
+            for _ in range(4):
+                gate_dev.copy_(gate_host, non_blocking=True)
+        say("cold start: two batches on one load")
+        cs.admit([0], tkn, mode="cpu_assisted")
+        cs.admit([0], tkn, mode="cpu_assisted")                    # same adapter again, its load still queued behind the gate
+        assert len(cs.tickets) == 1 and not cs.use_gpu_pipeline(20)
+        ys = [y.clone() for y in y0]
+        cs.finish_layer(cs.start_layer(x, 20, force="gpu"), x, 20, ys)     # the launch waits on the device for layer 20's rows
+        cs.admit([0], tkn, mode="cached")                          # the host waits for the rest of the load
+        assert cs.tickets == [] and cs.use_gpu_pipeline(0)
+        ys2 = [y.clone() for y in y0]
+        cs.finish_layer(cs.start_layer(x, 3), x, 3, ys2)
+        torch.cuda.synchronize()
+        for layer, out in ((20, ys), (3, ys2)):
+            for q, p in enumerate(NAMES):
+                want = _expected("gpu", weights, [0], scalings, tkn, layer, p, _bits(x), _bits(y0[q]))
+                err = np.abs(out[q].float().cpu().numpy() - want)
+                assert np.all(err <= ATOL + RTOL * np.abs(want)), (layer, p, float(err.max()))
+        cs.admit([1, 2, 3], tkn, mode="on_demand")                 # the pool has four slots
+        with pytest.raises(RuntimeError, match="no free slot"):
+            cs.admit([4], tkn, mode="on_demand")
+        cs.evict(2)
+        cs.admit([4], tkn, mode="on_demand")
+        ys3 = [y.clone() for y in y0]
+        cs.finish_layer(cs.start_layer(x, 31), x, 31, ys3)
+        torch.cuda.synchronize()
+        want = _expected("gpu", weights, [4], scalings, tkn, 31, "v", _bits(x), _bits(y0[2]))
+        err = np.abs(ys3[2].float().cpu().numpy() - want)
+        assert np.all(err <= ATOL + RTOL * np.abs(want))
+        with pytest.raises(KeyError):
+            cs.admit([7], tkn)
+    finally:
+        cs.stop_workers()
+        cpu.close()
